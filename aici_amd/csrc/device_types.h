@@ -1,0 +1,54 @@
+// Device-side scalar/vector types and conversions for gfx950.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hipattn {
+
+typedef _Float16 half_t;
+typedef __bf16 bf16_t;
+
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+template <typename T>
+struct Vec8;
+template <>
+struct Vec8<half_t> {
+  typedef half8_t type;
+};
+template <>
+struct Vec8<bf16_t> {
+  typedef bf16x8_t type;
+};
+
+template <typename T>
+__device__ __forceinline__ float to_float(T x) {
+  return (float)x;
+}
+
+// Round-to-nearest-even conversions; for bf16 this is gfx950's hardware
+// conversion, for fp16 v_cvt_f16_f32.
+template <typename T>
+__device__ __forceinline__ T from_float(float x) {
+  return (T)x;
+}
+
+// Bit-pattern helpers for building MFMA operands out of 32-bit registers.
+template <typename V, typename U>
+__device__ __forceinline__ V bit_cast(const U &u) {
+  static_assert(sizeof(V) == sizeof(U), "bit_cast size mismatch");
+  V v;
+  __builtin_memcpy(&v, &u, sizeof(V));
+  return v;
+}
+
+}  // namespace hipattn

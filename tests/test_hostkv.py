@@ -1,0 +1,190 @@
+"""Host side of the paged cache: the C++ core (through the C ABI) against hand-computed
+cases from blocks.rs / batch_info.rs and against the Python restatement, exactly."""
+import numpy as np
+import pytest
+
+from aici_amd import paged
+from aici_amd._lib import HipAttnError
+from oracle import hostkv as ref
+
+
+def test_allocation_order_and_slots_hand_case():
+    a = paged.BlockAllocator(16, 8)
+    assert a.get_num_free_blocks() == 8
+    a.alloc_seq(1, 40)  # 3 blocks: 0, 1, 2 (free list (0..n).rev() popped from the back)
+    a.alloc_seq(2, 16)  # 1 block: 3
+    assert a.num_allocated_blocks(1) == 3 and a.num_allocated_blocks(2) == 1
+    s1 = a.get_block_idxes(1, 40)
+    assert s1[0] == 0 and s1[15] == 15 and s1[16] == 16 and s1[39] == 2 * 16 + 7
+    assert list(a.get_block_idxes(2, 16)) == list(range(48, 64))
+    a.delete(1)  # frees 0,1,2 in that order -> pushed back; next pop is 2
+    assert a.get_num_free_blocks() == 7
+    a.alloc_seq(3, 1)
+    assert a.get_block_idxes(3, 1)[0] == 2 * 16
+
+
+def test_fork_copy_on_write_and_trim_hand_case():
+    a = paged.BlockAllocator(4, 10)
+    a.alloc_seq(1, 6)       # blocks 0,1
+    a.copy(1, 2, 6)         # fork: seq 2 shares blocks 0,1
+    assert a.get_num_free_blocks() == 8
+    # seq 2 appends token 7 (position 6 lives in shared block 1) -> COW copy of block 1
+    pairs = a.append_slots(2, 6, 7)
+    assert pairs == [(1, 2)]
+    assert list(a.get_block_idxes(2, 7)) == [0, 1, 2, 3, 8, 9, 10]
+    # seq 1 now owns block 1 alone -> no copy when it grows, new block when crossing a boundary
+    assert a.append_slots(1, 6, 9) == []
+    assert list(a.get_block_idxes(1, 9))[-1] == 3 * 4
+    a.trim(1, 4)            # keep one block
+    assert a.num_allocated_blocks(1) == 1
+    a.delete(1)
+    a.delete(2)
+    assert a.get_num_free_blocks() == 10
+
+
+def test_exhaustion_is_an_error_and_leaves_state_unchanged():
+    a = paged.BlockAllocator(16, 2)
+    with pytest.raises(HipAttnError, match="Out of memory! No free blocks"):
+        a.alloc_seq(1, 33)
+    assert a.get_num_free_blocks() == 2 and a.num_allocated_blocks(1) == 0
+    a.alloc_seq(1, 32)
+    with pytest.raises(HipAttnError, match="Out of memory"):
+        a.append_slots(1, 32, 33)
+    assert a.num_allocated_blocks(1) == 2
+    with pytest.raises(HipAttnError, match="unknown sequence"):
+        a.get_block_idxes(99, 1)
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_allocator_random_walk_matches_restatement(seed):
+    rng = np.random.default_rng(seed)
+    bs, nb = int(rng.choice([4, 16])), 64
+    a, r = paged.BlockAllocator(bs, nb), ref.BlockAllocator(bs, nb)
+    lens = {}
+    next_id = 1
+    for _ in range(200):
+        op = rng.integers(0, 5)
+        if op == 0 or not lens:
+            n = int(rng.integers(1, 5 * bs))
+            if r.get_num_free_blocks() < r.num_blocks(n):
+                continue
+            a.alloc_seq(next_id, n)
+            r.alloc_seq(next_id, n)
+            lens[next_id] = n
+            next_id += 1
+        elif op == 1:
+            s = int(rng.choice(list(lens)))
+            grow = int(rng.integers(1, 2 * bs))
+            if r.get_num_free_blocks() < r.num_blocks(lens[s] + grow) + 2:
+                continue
+            computed = int(rng.integers(max(0, lens[s] - bs), lens[s] + 1))
+            assert a.append_slots(s, computed, lens[s] + grow) == r.append_slots(s, computed, lens[s] + grow)
+            lens[s] += grow
+        elif op == 2:
+            s = int(rng.choice(list(lens)))
+            n = int(rng.integers(1, lens[s] + 1))
+            a.copy(s, next_id, n)
+            r.copy(s, next_id, n)
+            lens[next_id] = min(n, lens[s])
+            # a fork holds ceil(n/bs) blocks, so it can address up to that many tokens
+            lens[next_id] = min(r.num_allocated_blocks(next_id) * bs, lens[s])
+            next_id += 1
+        elif op == 3:
+            s = int(rng.choice(list(lens)))
+            n = int(rng.integers(0, lens[s] + 1))
+            a.trim(s, n)
+            r.trim(s, n)
+            if n == 0:
+                del lens[s]
+            else:
+                lens[s] = min(lens[s], r.num_allocated_blocks(s) * bs)
+        else:
+            s = int(rng.choice(list(lens)))
+            a.delete(s)
+            r.delete(s)
+            del lens[s]
+        assert a.get_num_free_blocks() == r.get_num_free_blocks()
+        for s, n in lens.items():
+            assert a.num_allocated_blocks(s) == r.num_allocated_blocks(s)
+            assert list(a.get_block_idxes(s, n)) == r.get_block_idxes(s, n)
+
+
+def _as_dict(bi: paged.BatchInfo) -> dict:
+    return dict(tokens=bi.tokens.tolist(), positions=bi.positions.tolist(), slot_mapping=bi.slot_mapping.tolist(),
+                logit_idxs=bi.logit_idxs.tolist(), seq_ids=bi.seq_ids, seqlens_q=bi.seqlens_q.tolist(),
+                seqlens_k=bi.seqlens_k.tolist(), max_seqlen_q=bi.max_seqlen_q, max_seqlen_k=bi.max_seqlen_k,
+                gather_mapping=bi.gather_mapping.tolist(), seqlen_multi=bi.seqlen_multi, q_multi=bi.q_multi,
+                paged_block_tables=bi.paged_block_tables.flatten().tolist(),
+                paged_max_blocks=bi.paged_block_tables.shape[1], paged_context_lens=bi.paged_context_lens.tolist(),
+                paged_block_size=bi.paged_block_size, paged_max_context_len=bi.paged_max_context_len)
+
+
+def test_batch_builder_hand_case_multi_first_ordering():
+    bs = 4
+    a = paged.BlockAllocator(bs, 16)
+    a.alloc_seq(10, 5)   # decode row: blocks 0,1 ; context 5
+    a.alloc_seq(11, 6)   # prompt of 6: blocks 2,3
+    a.alloc_seq(12, 9)   # decode row: blocks 4,5,6 ; context 9
+    b = paged.BatchInfoBuilder(bs, 128, paged_attn_kernel_v=1)
+    b.sched_out(a, 10, [100, 101, 102, 103, 104], 4)
+    b.sched_out(a, 11, [200, 201, 202, 203, 204, 205], 0)
+    b.sched_out(a, 12, list(range(300, 309)), 9)  # nothing new: recompute the last token
+    bi = b.finish()
+    assert bi.seq_ids == [11, 10, 12]                      # multi-token entry first, singles keep order
+    assert bi.tokens.tolist() == [200, 201, 202, 203, 204, 205, 104, 308]
+    assert bi.positions.tolist() == [0, 1, 2, 3, 4, 5, 4, 8]
+    assert bi.slot_mapping.tolist() == [8, 9, 10, 11, 12, 13, 4, 24]
+    assert bi.logit_idxs.tolist() == [5, 6, 7]
+    assert bi.seqlens_q.tolist() == [0, 6] and bi.seqlens_k.tolist() == [0, 6]
+    assert bi.gather_mapping.tolist() == [8, 9, 10, 11, 12, 13]
+    assert bi.q_multi == 6 and bi.seqlen_multi == 1
+    assert bi.paged_context_lens.tolist() == [5, 9] and bi.paged_max_context_len == 9
+    assert bi.paged_block_tables.tolist() == [[0, 1, 0], [4, 5, 6]]   # zero padded
+    # CPU-build behaviour: everything on the varlen path, original order
+    b0 = paged.BatchInfoBuilder(bs, 128, paged_attn_kernel_v=0)
+    b0.sched_out(a, 10, [100, 101, 102, 103, 104], 4)
+    b0.sched_out(a, 11, [200, 201, 202, 203, 204, 205], 0)
+    bi0 = b0.finish()
+    assert bi0.seq_ids == [10, 11] and bi0.seqlen_multi == 2 and bi0.q_multi == 7
+    assert bi0.seqlens_q.tolist() == [0, 1, 7] and bi0.seqlens_k.tolist() == [0, 5, 11]
+    assert bi0.paged_block_tables.numel() == 0
+
+
+@pytest.mark.parametrize("seed", range(4))
+@pytest.mark.parametrize("paged_v", [0, 1])
+def test_batch_builder_matches_restatement(seed, paged_v):
+    rng = np.random.default_rng(100 + seed)
+    bs = 16
+    a, r = paged.BlockAllocator(bs, 256), ref.BlockAllocator(bs, 256)
+    b = paged.BatchInfoBuilder(bs, 4096, paged_v)
+    entries = []
+    for sid in range(1, 12):
+        n = int(rng.integers(1, 200))
+        toks = rng.integers(0, 32000, size=n).tolist()
+        a.alloc_seq(sid, n)
+        r.alloc_seq(sid, n)
+        computed = int(rng.choice([0, n, n - 1, max(0, n - 5)]))
+        b.sched_out(a, sid, toks, computed)
+        entries.append(ref.sched_entry(r, sid, toks, computed))
+    got = _as_dict(b.finish())
+    want = ref.build_batch(entries, bs, 4096, paged_v)
+    assert got == want
+
+
+def test_builder_errors():
+    b = paged.BatchInfoBuilder(16, 8, 1)
+    with pytest.raises(HipAttnError, match="no entries"):
+        b.finish()
+    b.add_entry(1, [9], [5], list(range(10)))
+    with pytest.raises(HipAttnError, match="max_model_len"):
+        b.finish()
+    b2 = paged.BatchInfoBuilder(16, 100, 1)
+    b2.add_entry(1, [2], [5], [3, 4, 5])  # first slot of the context is not block-aligned
+    with pytest.raises(HipAttnError, match="not block-aligned"):
+        b2.finish()
+
+
+def test_cache_geometry():
+    import torch
+    assert paged.cache_x(torch.float16) == 8 and paged.cache_x(torch.bfloat16) == 8 and paged.cache_x(torch.float32) == 4
+    assert paged.cache_block_bytes(16, 8, 128, 32, torch.bfloat16) == ref.cache_block_bytes(16, 8, 128, 32, 2) == 2 * 16 * 8 * 128 * 2 * 32
