@@ -7,6 +7,7 @@ from __future__ import annotations
 import math
 from typing import Optional, Tuple
 
+import numpy as np
 import torch
 
 from . import kernels
@@ -28,8 +29,8 @@ class RotaryEmbedding:
     @staticmethod
     def build_table(rotary_dim: int, rope_theta: float, max_len: int, dtype: torch.dtype) -> torch.Tensor:
         # theta_i = 1 / rope_theta^(i / rotary_dim), i even, in f32 (mod.rs:44-47)
-        idx = torch.arange(0, rotary_dim, 2, dtype=torch.float32)
-        theta = 1.0 / torch.pow(torch.tensor(float(rope_theta), dtype=torch.float32), idx / float(rotary_dim))
+        expo = np.arange(0, rotary_dim, 2, dtype=np.float32) / np.float32(rotary_dim)
+        theta = torch.from_numpy(np.float32(1.0) / np.power(np.float32(rope_theta), expo, dtype=np.float32))
         idx_theta = torch.arange(max_len, dtype=torch.float32).reshape(max_len, 1).matmul(theta.reshape(1, -1))
         return torch.cat([idx_theta.cos().to(dtype), idx_theta.sin().to(dtype)], dim=-1).contiguous()
 

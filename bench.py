@@ -1,0 +1,168 @@
+"""Benchmark of the rLLM attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Headline (`value`): paged decode attention over the benchmark's decode configuration
+(64 sequences, contexts U[512,4096], 32 q / 8 kv heads, d 128, bf16, block size 16, tables from
+a shuffled 20k-block pool) as algorithmic HBM GB/s, with inputs resident in HBM.  One step = one
+`paged_attention_v1` call over the batch.  The same line also carries the prefill leg
+(`prefill`: 8 x 4096 GQA causal varlen prefill, TFLOP/s against the bf16 MFMA peak) and the CPU
+baseline (`cpu_baseline`: the oracle, i.e. rLLM's CPU reference route restated in torch-CPU,
+timed on a bounded sample of the same workload on this box's host cores).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
+
+
+def event_times_ms(fn, steps: int, stream) -> list:
+    """Per-launch durations from HIP events recorded on the stream the kernels run on."""
+    import torch
+
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in evs:
+        a.record(stream)
+        fn()
+        b.record(stream)
+    torch.cuda.synchronize()
+    return [a.elapsed_time(b) for a, b in evs]
+
+
+def cpu_baseline_decode(c_cpu, rows, threads: int) -> dict:
+    """The oracle (gather_cached_kv -> repeat_kv -> Lq=1 varlen SDPA in fp32, the route rLLM's CPU
+    build takes) on a sample of the sequences."""
+    import torch
+
+    from oracle import refkernels as ref
+
+    torch.set_num_threads(threads)
+    q = c_cpu.q[rows].float()
+    kc, vc = c_cpu.key_cache.float(), c_cpu.value_cache.float()
+    bt, cl = c_cpu.block_tables[rows], c_cpu.context_lens[rows]
+    reps, dt = 0, 0.0
+    t0 = time.perf_counter()
+    while dt < 12.0:  # a bounded sample: about 12 s of CPU work
+        ref.paged_attention(q, kc, vc, c_cpu.num_kv_heads, c_cpu.scale, bt, cl, 16)
+        reps += 1
+        dt = time.perf_counter() - t0
+    dt /= reps
+    elt = c_cpu.q.element_size()
+    tokens = int(cl.sum())
+    nbytes = tokens * 2 * c_cpu.num_kv_heads * c_cpu.q.shape[2] * elt + 2 * len(rows) * q.shape[1] * q.shape[2] * elt
+    return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{len(rows)} of {c_cpu.q.shape[0]} sequences ({tokens} context tokens), {reps} passes of {dt:.2f} s; "
+                      "bytes counted as for the GPU (bf16 K/V once per kv head)"}
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the attention path has no cross-GPU step in this build "
+                 "(run with --gpus 1)")
+    import torch
+
+    from aici_amd import kernels as K
+    from aici_amd import workloads as W
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream(dev)
+
+    # ---- decode leg (headline) ------------------------------------------------------------
+    c_cpu = W.config2()
+    c = c_cpu.to(dev)
+    out = torch.empty_like(c.q)
+
+    def decode_step():
+        K.paged_attention_v1(out, c.q, c.key_cache, c.value_cache, c.num_kv_heads, c.scale, c.block_tables,
+                             c.context_lens, 16, c.max_ctx)
+
+    for _ in range(args.warmup):
+        decode_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        decode_step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    launch_ms = event_times_ms(decode_step, args.steps, stream)
+    avg_launch_ms = sum(launch_ms) / len(launch_ms)
+    nbytes = c_cpu.algorithmic_bytes()
+    value = nbytes / (wall_ms * 1e-3) / 1e9
+    achieved = nbytes / (avg_launch_ms * 1e-3) / 1e9
+
+    line = {
+        "metric": "prefill attn TFLOP/s + paged-decode attn HBM GB/s (1 GPU, % roofline)",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "paged decode attention: 64 seqs, ctx U[512,4096] (seed 2), 32 q / 8 kv heads, "
+                               "d 128, bf16, block 16, tables from a shuffled 20k-block pool",
+                   "algorithmic_bytes_per_step": nbytes,
+                   "context_tokens": int(c_cpu.context_lens.sum())},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "paged_decode_kernel (+ reduce) per step, HIP events",
+                     "avg_launch_us": round(avg_launch_ms * 1e3, 2)},
+    }
+
+    # ---- prefill leg ------------------------------------------------------------------------
+    if not args.no_prefill:
+        p = W.config3(1.0, device=dev)
+
+        def prefill_step():
+            K.flash_attn_varlen(p.q, p.k, p.v, p.cu_q, p.cu_k, p.max_q, p.max_k, p.scale, True)
+
+        psteps = max(3, min(args.steps, 20))
+        for _ in range(max(1, min(args.warmup, 5))):
+            prefill_step()
+        torch.cuda.synchronize()
+        pl = event_times_ms(prefill_step, psteps, stream)
+        pms = sum(pl) / len(pl)
+        tflops = p.flops() / (pms * 1e-3) / 1e12
+        line["prefill"] = {
+            "value": round(tflops, 1), "unit": "TFLOP/s", "ms_per_step": round(pms, 4), "steps": psteps,
+            "config": {"workload": "varlen causal prefill: 8 x 4096 tokens, 32 q / 8 kv heads, d 128, bf16, N(0,1)",
+                       "algorithmic_flops_per_step": p.flops()},
+            "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                         "kernel": "prefill_varlen_kernel, HIP events"},
+        }
+        del p
+
+    # ---- CPU baseline: the reference's CPU route on this box's host cores ------------------------
+    if not args.no_cpu_baseline:
+        threads = min(os.cpu_count() or 1, 16)
+        line["cpu_baseline"] = cpu_baseline_decode(c_cpu, list(range(0, 64, 2)), threads)
+
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

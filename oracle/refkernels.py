@@ -116,6 +116,8 @@ def varlen_attn_fp64(q, k, v, seqlens_q, seqlens_k, softmax_scale: float, causal
     out = torch.zeros(q.shape, dtype=torch.float64)
     for i in range(len(sq) - 1):
         lq, lk = sq[i + 1] - sq[i], sk[i + 1] - sk[i]
+        if lq == 0 or lk == 0:
+            continue  # no rows, or rows without any key: zeros
         qi = q[sq[i]:sq[i] + lq].double()
         ki = k[sk[i]:sk[i] + lk].double()
         vi = v[sk[i]:sk[i] + lk].double()
@@ -146,6 +148,8 @@ def flash_numerics_model(q, k, v, seqlens_q, seqlens_k, softmax_scale: float, ca
     out = torch.zeros(q.shape, dtype=dt)
     for i in range(len(sq) - 1):
         lq, lk = sq[i + 1] - sq[i], sk[i + 1] - sk[i]
+        if lq == 0 or lk == 0:
+            continue
         qi, ki, vi = q[sq[i]:sq[i] + lq].float(), k[sk[i]:sk[i] + lk].float(), v[sk[i]:sk[i] + lk].float()
         rows = torch.arange(lq).reshape(lq, 1)
         cols = torch.arange(lk).reshape(1, lk)
@@ -200,8 +204,11 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
 def rotary_table(rotary_dim: int, rope_theta: float, max_len: int, dtype: torch.dtype) -> torch.Tensor:
     """mod.rs:41-60 `RotaryEmbedding::new`: theta_i = 1/rope_theta^(i/rot) (f32, i even),
     idx_theta = pos (x) theta, cat(cos, sin) cast to the model dtype -> [max_len, rot]."""
-    theta = torch.tensor([1.0 / (float(rope_theta) ** (i / float(rotary_dim))) for i in range(0, rotary_dim, 2)],
-                         dtype=torch.float32)
+    import numpy as np
+    f32 = np.float32
+    # every operation in f32, as the Rust expression `1f32 / rope_theta.powf(i as f32 / rotary_dim as f32)`
+    theta = torch.tensor([float(f32(1.0) / np.power(f32(rope_theta), f32(i) / f32(rotary_dim), dtype=f32))
+                          for i in range(0, rotary_dim, 2)], dtype=torch.float32)
     idx_theta = torch.arange(max_len, dtype=torch.float32).reshape(max_len, 1).matmul(theta.reshape(1, -1))
     return torch.cat([idx_theta.cos().to(dtype), idx_theta.sin().to(dtype)], dim=-1).contiguous()
 

@@ -1,0 +1,127 @@
+"""reshape_and_cache / gather_cached_kv / copy_blocks / swap_blocks through the C ABI against
+the oracle: bit-exact."""
+import pytest
+import torch
+
+from aici_amd import kernels as K
+from aici_amd import workloads as W
+from aici_amd._lib import HipAttnError
+from oracle import refkernels as ref
+from tests.common import make_cache
+
+pytestmark = pytest.mark.gpu
+
+
+def bits(t: torch.Tensor) -> torch.Tensor:
+    return t.cpu().contiguous().view(torch.int16 if t.element_size() == 2 else torch.int32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("slot_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("strided", [False, True])
+def test_reshape_and_cache_and_gather_bit_exact(device, dtype, slot_dtype, strided):
+    g = torch.Generator().manual_seed(1)
+    T, H, d, bs, nb = 150, 5, 80, 16, 24
+    if strided:  # k and v as chunks of a fused [T, 3, H, d] projection, as rLLM's Phi layer passes them
+        qkv = torch.randn((T, 3, H, d), generator=g).to(dtype)
+        key, value = qkv[:, 1], qkv[:, 2]
+    else:
+        key = torch.randn((T, H, d), generator=g).to(dtype)
+        value = torch.randn((T, H, d), generator=g).to(dtype)
+    kc, vc = make_cache(nb, H, d, bs, dtype, fill=-3.0)
+    slots = torch.randperm(nb * bs, generator=g)[:T].to(slot_dtype)
+    slots[7] = -1
+    slots[T - 1] = -5
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    ref.reshape_and_cache(key, value, kc_ref, vc_ref, slots)
+    kd, vd = kc.to(device), vc.to(device)
+    if strided:
+        qkv_d = qkv.to(device)
+        key_d, value_d = qkv_d[:, 1], qkv_d[:, 2]
+    else:
+        key_d, value_d = key.to(device), value.to(device)
+    if slot_dtype == torch.int64:
+        K.reshape_and_cache(key_d, value_d, kd, vd, slots.to(device))
+    else:  # int32 straight through the ABI (the Python mirror widens; the ABI accepts both)
+        from aici_amd.kernels import _desc, _stream, call
+        call("hipattn_reshape_and_cache", _desc(key_d), _desc(value_d), _desc(kd), _desc(vd),
+             _desc(slots.to(device)), _stream(key_d))
+    assert torch.equal(bits(kd), bits(kc_ref)) and torch.equal(bits(vd), bits(vc_ref))
+    valid = slots >= 0
+    n = int(valid.sum())
+    ko = torch.zeros((n, H, d), dtype=dtype, device=device)
+    vo = torch.zeros_like(ko)
+    gslots = slots[valid].to(torch.int32 if slot_dtype == torch.int32 else torch.int64)
+    K.gather_cached_kv(ko, vo, kd, vd, gslots.to(device))
+    assert torch.equal(bits(ko), bits(key[valid])) and torch.equal(bits(vo), bits(value[valid]))
+
+
+def test_config1_scatter_bit_exact(device):
+    p, extra = W.config1()
+    nb = extra["pool_blocks"]
+    kc, vc = make_cache(nb, 32, 128, 16, torch.float16, fill=0.5)
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    ref.reshape_and_cache(p.k, p.v, kc_ref, vc_ref, extra["slot_mapping"])
+    kd, vd = kc.to(device), vc.to(device)
+    K.reshape_and_cache(p.k.to(device), p.v.to(device), kd, vd, extra["slot_mapping"].to(device))
+    assert torch.equal(bits(kd), bits(kc_ref)) and torch.equal(bits(vd), bits(vc_ref))
+    # 80 of the 128 blocks are used; the others still hold the fill value
+    used = torch.unique(extra["slot_mapping"] // 16)
+    assert used.numel() == 80
+    mask = torch.ones(nb, dtype=torch.bool)
+    mask[used.long()] = False
+    assert torch.all(kd.cpu()[mask] == 0.5) and torch.all(vd.cpu()[mask] == 0.5)
+
+
+def test_empty_and_out_of_range(device):
+    kc, vc = make_cache(4, 2, 64, 16, torch.bfloat16, fill=1.0)
+    kd, vd = kc.to(device), vc.to(device)
+    e = torch.zeros((0, 2, 64), dtype=torch.bfloat16, device=device)
+    K.reshape_and_cache(e, e, kd, vd, torch.zeros((0,), dtype=torch.int64, device=device))
+    K.gather_cached_kv(e, e, kd, vd, torch.zeros((0,), dtype=torch.int32, device=device))
+    # a slot beyond the cache is dropped instead of written out of bounds
+    one = torch.ones((1, 2, 64), dtype=torch.bfloat16, device=device) * 9
+    K.reshape_and_cache(one, one, kd, vd, torch.tensor([4 * 16 + 3], dtype=torch.int64, device=device))
+    torch.cuda.synchronize()
+    assert torch.all(kd.cpu() == 1.0) and torch.all(vd.cpu() == 1.0)
+
+
+def test_argument_errors(device):
+    kc, vc = make_cache(4, 2, 64, 16, torch.float16)
+    kd, vd = kc.to(device), vc.to(device)
+    k = torch.zeros((3, 2, 64), dtype=torch.float16, device=device)
+    s = torch.zeros((3,), dtype=torch.int64, device=device)
+    with pytest.raises(HipAttnError, match="dtype must match"):
+        K.reshape_and_cache(k.to(torch.bfloat16), k.to(torch.bfloat16), kd, vd, s)
+    with pytest.raises(HipAttnError, match="heads of size"):
+        K.reshape_and_cache(k[:, :1], k[:, :1], kd, vd, s)
+    with pytest.raises(HipAttnError, match="slot_mapping has"):
+        K.reshape_and_cache(k, k, kd, vd, s[:2])
+    with pytest.raises(HipAttnError, match="GPU tensor"):
+        K.reshape_and_cache(k.cpu(), k, kd, vd, s)
+
+
+def test_copy_blocks_and_swap_blocks(device):
+    g = torch.Generator().manual_seed(5)
+    layers = 3
+    caches = [make_cache(10, 2, 64, 16, torch.bfloat16, gen=g) for _ in range(layers)]
+    kcs = [c[0].clone() for c in caches]
+    vcs = [c[1].clone() for c in caches]
+    mapping = {1: [4, 5], 2: [0], 9: [8]}
+    kd = [k.to(device) for k in kcs]
+    vd = [v.to(device) for v in vcs]
+    K.copy_blocks(kd, vd, mapping)
+    ref.copy_blocks(kcs, vcs, mapping)
+    for l in range(layers):
+        assert torch.equal(bits(kd[l]), bits(kcs[l])) and torch.equal(bits(vd[l]), bits(vcs[l]))
+    K.copy_blocks(kd, vd, {})  # no pairs: no launch
+    # swap out blocks 3,4 to a pinned host cache at 0,1 and back in at 6,7
+    host = torch.zeros((4,) + tuple(kd[0].shape[1:]), dtype=torch.bfloat16).pin_memory()
+    K.swap_blocks(kd[0], host, {3: 0, 4: 1})
+    torch.cuda.synchronize()
+    assert torch.equal(bits(host[0]), bits(kcs[0][3])) and torch.equal(bits(host[1]), bits(kcs[0][4]))
+    K.swap_blocks(host, kd[0], {0: 6, 1: 7})
+    torch.cuda.synchronize()
+    assert torch.equal(bits(kd[0][6]), bits(kcs[0][3])) and torch.equal(bits(kd[0][7]), bits(kcs[0][4]))
+    with pytest.raises(HipAttnError, match="out of range"):
+        K.swap_blocks(kd[0], host, {3: 99})

@@ -1,0 +1,181 @@
+"""Paged decode attention through the C ABI against the oracle (gather + Lq=1 varlen SDPA,
+the way rLLM's CPU build computes single-token rows).  Gates: max-abs error <= 2e-2 (bf16),
+<= 5e-3 (fp16) against the fp32 oracle on the same rounded inputs."""
+import numpy as np
+import pytest
+import torch
+
+from aici_amd import kernels as K
+from aici_amd import workloads as W
+from aici_amd._lib import HipAttnError
+from oracle import refkernels as ref
+from tests.common import TOL
+
+pytestmark = pytest.mark.gpu
+
+
+def run_v1(c: W.DecodeInputs, device, alibi=None):
+    d = c.to(device)
+    out = torch.full_like(d.q, float("nan"))
+    K.paged_attention_v1(out, d.q, d.key_cache, d.value_cache, c.num_kv_heads, c.scale, d.block_tables,
+                         d.context_lens, 16, c.max_ctx, alibi.to(device) if alibi is not None else None)
+    return out.cpu()
+
+
+def oracle(c: W.DecodeInputs, alibi=None, rows=None):
+    q, bt, cl = c.q, c.block_tables, c.context_lens
+    if rows is not None:
+        q, bt, cl = q[rows], bt[rows], cl[rows]
+    return ref.paged_attention(q.float(), c.key_cache.float(), c.value_cache.float(), c.num_kv_heads, c.scale, bt,
+                               cl, 16, alibi)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("heads", [(32, 8, 128), (32, 32, 80), (8, 8, 64), (16, 1, 96), (40, 2, 112), (4, 4, 256)])
+def test_matches_oracle_over_head_shapes(device, dtype, heads):
+    Hq, Hkv, d = heads
+    c = W.decode_inputs(11, 9, 1, 1500, Hq, Hkv, d, dtype, 1024)
+    got = run_v1(c, device)
+    want = oracle(c)
+    assert not torch.isnan(got).any()
+    assert (got.float() - want).abs().max().item() <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_context_edge_lengths_and_stale_cache_contents(device, dtype):
+    # Contexts around block and partition boundaries, including 0; every cache slot that no
+    # context covers holds NaN, as an uninitialised (torch.empty) cache may.
+    lens = [0, 1, 15, 16, 17, 31, 32, 33, 127, 128, 129, 255, 256, 257, 511, 512, 513, 1023, 1025]
+    S = len(lens)
+    c = W.decode_inputs(12, S, 1, 2, 32, 8, 128, dtype, 700)
+    ctx = np.array(lens, dtype=np.int32)
+    nblk = (ctx + 15) // 16
+    perm = np.random.default_rng(3).permutation(700)
+    tables = np.zeros((S, int(nblk.max())), dtype=np.int32)
+    covered = torch.zeros((700, 16), dtype=torch.bool)
+    pos = 0
+    for s in range(S):
+        tables[s, :nblk[s]] = perm[pos:pos + nblk[s]]
+        for t in range(ctx[s]):
+            covered[tables[s, t // 16], t % 16] = True
+        pos += nblk[s]
+    c.block_tables, c.context_lens, c.max_ctx = torch.from_numpy(tables), torch.from_numpy(ctx), int(ctx.max())
+    kc, vc = c.key_cache, c.value_cache
+    kc.permute(0, 3, 1, 2, 4)[~covered] = float("nan")
+    vc.permute(0, 3, 1, 2)[~covered] = float("nan")
+    got = run_v1(c, device)
+    kc.permute(0, 3, 1, 2, 4)[~covered] = 0.0   # the oracle never reads them; avoid NaN*0 in its gathers
+    vc.permute(0, 3, 1, 2)[~covered] = 0.0
+    want = oracle(c)
+    assert not torch.isnan(got).any()
+    assert torch.all(got[0] == 0)  # empty context -> zeros
+    assert (got.float() - want).abs().max().item() <= TOL[dtype]
+
+
+def test_single_partition_path_and_many_partitions_agree_with_oracle(device):
+    # S large -> one partition per sequence; S = 1 -> the context is split many ways.
+    big = W.decode_inputs(13, 300, 100, 400, 8, 2, 128, torch.float16, 8000)
+    assert (run_v1(big, device).float() - oracle(big)).abs().max().item() <= TOL[torch.float16]
+    one = W.decode_inputs(14, 1, 4000, 4096, 32, 8, 128, torch.float16, 300)
+    assert (run_v1(one, device).float() - oracle(one)).abs().max().item() <= TOL[torch.float16]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_v2_entry_with_caller_workspaces(device, dtype):
+    c = W.decode_inputs(15, 6, 200, 1400, 32, 8, 128, dtype, 600)
+    d = c.to(device)
+    want = oracle(c)
+    for part_tokens in (512, 96):
+        P = (c.max_ctx + part_tokens - 1) // part_tokens
+        S, Hq, hd = c.q.shape
+        exp_sums = torch.empty((S, Hq, P), dtype=torch.float32, device=device)
+        max_logits = torch.empty_like(exp_sums)
+        tmp_out = torch.empty((S, Hq, P, hd), dtype=dtype, device=device)
+        out = torch.empty_like(d.q)
+        K.paged_attention_v2(out, exp_sums, max_logits, tmp_out, d.q, d.key_cache, d.value_cache, 8, c.scale,
+                             d.block_tables, d.context_lens, 16, c.max_ctx)
+        assert (out.cpu().float() - want).abs().max().item() <= TOL[dtype]
+    # the reference's partials: max_logits are natural-log maxima of the scaled scores
+    s0 = 0
+    ctx0 = int(c.context_lens[s0])
+    slots = torch.tensor(W.slots_for(c.block_tables[s0].tolist(), min(ctx0, 96)), dtype=torch.int32)
+    kk = torch.empty((len(slots), 8, 128), dtype=dtype)
+    vv = torch.empty_like(kk)
+    ref.gather_cached_kv(kk, vv, c.key_cache, c.value_cache, slots)
+    logits = (kk[:, 0].float() @ c.q[s0, 0].float()) * c.scale
+    assert abs(max_logits[s0, 0, 0].item() - logits.max().item()) < 2e-2
+
+
+def test_alibi_and_strided_query(device):
+    dtype = torch.float16
+    c = W.decode_inputs(16, 5, 10, 600, 32, 32, 80, dtype, 300)
+    slopes = torch.tensor([2.0 ** (-(i + 1) / 4) for i in range(32)], dtype=torch.float32)
+    got = run_v1(c, device, slopes)
+    want = oracle(c, slopes)
+    assert (got.float() - want).abs().max().item() <= TOL[dtype]
+    # q as a chunk of a fused [S, 3, H, d] projection (row stride 3*H*d), as Phi passes it
+    d = c.to(device)
+    fused = torch.zeros((5, 3, 32, 80), dtype=dtype, device=device)
+    fused[:, 0] = d.q
+    out = torch.empty_like(d.q)
+    K.paged_attention_v1(out, fused[:, 0], d.key_cache, d.value_cache, 32, c.scale, d.block_tables, d.context_lens,
+                         16, c.max_ctx)
+    assert (out.cpu().float() - oracle(c)).abs().max().item() <= TOL[dtype]
+
+
+def test_invariant_under_block_permutation_and_equals_prefill_last_row(device):
+    dtype = torch.bfloat16
+    c = W.decode_inputs(17, 4, 50, 700, 32, 8, 128, dtype, 256)
+    got = run_v1(c, device)
+    perm = torch.randperm(256, generator=torch.Generator().manual_seed(1))
+    kc2, vc2 = torch.empty_like(c.key_cache), torch.empty_like(c.value_cache)
+    kc2[perm] = c.key_cache
+    vc2[perm] = c.value_cache
+    c2 = W.DecodeInputs(c.q, kc2, vc2, perm[c.block_tables.long()].to(torch.int32), c.context_lens, c.max_ctx,
+                        c.scale, 8)
+    assert torch.equal(run_v1(c2, device), got)  # same arithmetic in the same order
+    # the decode row equals the last row of a causal prefill over the same keys
+    s = 1
+    ctx = int(c.context_lens[s])
+    slots = torch.tensor(W.slots_for(c.block_tables[s].tolist(), ctx), dtype=torch.int32)
+    kk = torch.empty((ctx, 8, 128), dtype=dtype)
+    vv = torch.empty_like(kk)
+    ref.gather_cached_kv(kk, vv, c.key_cache, c.value_cache, slots)
+    qq = torch.zeros((ctx, 32, 128), dtype=dtype)
+    qq[-1] = c.q[s]
+    cu = W.offsets([ctx]).to(device)
+    pre = K.flash_attn_varlen(qq.to(device), kk.to(device), vv.to(device), cu, cu, ctx, ctx, c.scale, True)
+    assert (pre[-1].cpu().float() - got[s].float()).abs().max().item() <= 2e-2
+
+
+def test_config2_full_size(device):
+    """The benchmark's decode configuration at full size: every sequence against the oracle."""
+    c = W.config2()
+    assert c.q.shape == (64, 32, 128) and c.key_cache.shape == (20000, 8, 16, 16, 8)
+    got = run_v1(c, device)
+    assert not torch.isnan(got).any()
+    rows = list(range(0, 64, 3))  # 22 of the 64 sequences through the (slow) oracle
+    want = oracle(c, rows=rows)
+    assert (got[rows].float() - want).abs().max().item() <= TOL[torch.bfloat16]
+    # size-independent property on all 64: attention output is a convex combination of the
+    # context's V rows, so each coordinate lies within the range of that kv head's values
+    assert got.float().abs().max().item() <= c.value_cache.float().abs().max().item()
+
+
+def test_argument_errors(device):
+    c = W.decode_inputs(18, 2, 5, 40, 8, 2, 128, torch.float16, 16).to(device)
+    out = torch.empty_like(c.q)
+    args = (c.key_cache, c.value_cache, 2, c.scale, c.block_tables, c.context_lens)
+    with pytest.raises(HipAttnError, match="unsupported block size 32"):
+        K.paged_attention_v1(out, c.q, *args, 32, c.max_ctx)
+    with pytest.raises(HipAttnError, match="unsupported data type f32"):
+        K.paged_attention_v1(out.float(), c.q.float(), c.key_cache.float(), c.value_cache.float(), 2, c.scale,
+                             c.block_tables, c.context_lens, 16, c.max_ctx)
+    with pytest.raises(HipAttnError, match="not divisible"):
+        K.paged_attention_v1(out, c.q, c.key_cache, c.value_cache, 3, c.scale, c.block_tables, c.context_lens, 16,
+                             c.max_ctx)
+    with pytest.raises(HipAttnError, match="block-table columns"):
+        K.paged_attention_v1(out, c.q, *args, 16, 16 * c.block_tables.size(1) + 1)
+    bad = torch.empty((2, 8, 72), dtype=torch.float16, device=c.q.device)
+    with pytest.raises(HipAttnError):
+        K.paged_attention_v1(bad, bad, *args, 16, c.max_ctx)

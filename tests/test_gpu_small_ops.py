@@ -1,0 +1,183 @@
+"""rotary_embedding, rms_norm, activations, bias_argmax and the runtime plumbing through the
+C ABI against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from aici_amd import attn, kernels as K
+from aici_amd import workloads as W
+from aici_amd._lib import HipAttnError
+from oracle import aici
+from oracle import refkernels as ref
+
+pytestmark = pytest.mark.gpu
+
+
+def ulp_diff16(a: torch.Tensor, b: torch.Tensor) -> int:
+    """Largest distance in representable values between two fp16/bf16 tensors."""
+    def key(t):
+        i = t.cpu().contiguous().view(torch.int16).to(torch.int32)
+        return torch.where(i < 0, -(i & 0x7FFF), i)
+    return int((key(a) - key(b)).abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(32, 8, 128, 128), (32, 32, 80, 32), (4, 1, 64, 64)])  # Hq, Hkv, d, rot
+@pytest.mark.parametrize("neox", [True, False])
+def test_rotary_matches_oracle(device, dtype, shape, neox):
+    Hq, Hkv, d, rot = shape
+    g = torch.Generator().manual_seed(3)
+    T, max_pos = 37, 512
+    table = ref.rotary_table(rot, 10000.0, max_pos, dtype)
+    assert torch.equal(table, attn.RotaryEmbedding.build_table(rot, 10000.0, max_pos, dtype))
+    q = torch.randn((T, Hq * d), generator=g).to(dtype)
+    k = torch.randn((T, Hkv * d), generator=g).to(dtype)
+    pos = torch.randint(0, max_pos, (T,), generator=g, dtype=torch.int64)
+    pos[0] = 0
+    qd, kd = q.clone().to(device), k.clone().to(device)
+    K.rotary_embedding(pos.to(device), qd, kd, d, table.to(device), neox)
+    ref.rotary_embedding(pos, q, k, d, table, neox)
+    if dtype == torch.float32:
+        # the reference's own self-check tolerance for this op is 1e-5 (llm/mod.rs:104-105)
+        assert (qd.cpu() - q).abs().max().item() <= 1e-6 and (kd.cpu() - k).abs().max().item() <= 1e-6
+    else:  # same rounding points as the oracle's per-op arithmetic: bit-exact
+        assert torch.equal(qd.cpu().view(torch.int16), q.view(torch.int16))
+        assert torch.equal(kd.cpu().view(torch.int16), k.view(torch.int16))
+
+
+def test_rotary_strided_rows_and_int32_positions(device):
+    g = torch.Generator().manual_seed(4)
+    T, H, d = 9, 4, 64
+    table = ref.rotary_table(d, 10000.0, 64, torch.float16)
+    big = torch.randn((T, 3 * H * d), generator=g).to(torch.float16)
+    q, k = big[:, :H * d], big[:, H * d:2 * H * d]  # row stride 3*H*d
+    pos = torch.arange(T, dtype=torch.int32)
+    bd = big.clone().to(device)
+    K.rotary_embedding(pos.to(device), bd[:, :H * d], bd[:, H * d:2 * H * d], d, table.to(device), True)
+    qc, kc = q.clone().contiguous(), k.clone().contiguous()
+    ref.rotary_embedding(pos, qc, kc, d, table, True)
+    out = bd.cpu()
+    assert torch.equal(out[:, :H * d], qc) and torch.equal(out[:, H * d:2 * H * d], kc)
+    assert torch.equal(out[:, 2 * H * d:], big[:, 2 * H * d:])  # the v third is untouched
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("hidden", [4096, 2560, 100])
+def test_rms_norm_and_fused(device, dtype, hidden):
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn((17, hidden), generator=g) * 3).to(dtype)
+    w = (1 + 0.1 * torch.randn((hidden,), generator=g)).to(dtype)
+    out = torch.empty_like(x).to(device)
+    K.rms_norm(out, x.to(device), w.to(device), 1e-5)
+    want = ref.rms_norm(x, w, 1e-5)
+    if dtype == torch.float32:
+        assert (out.cpu() - want).abs().max().item() <= 2e-6 * want.abs().max().item()
+    else:
+        # The fp32 reduction order differs, which can move the first rounding by one value; the
+        # multiply by a weight above 1 can stretch that to two values of the result.
+        assert ulp_diff16(out, want) <= 2
+        assert (out.cpu() == want).float().mean().item() > 0.995
+    r = torch.randn((17, hidden), generator=g).to(dtype)
+    xi, ri = x.clone(), r.clone()
+    ref.fused_add_rms_norm(xi, ri, w, 1e-5)
+    xd, rd = x.clone().to(device), r.clone().to(device)
+    K.fused_add_rms_norm(xd, rd, w.to(device), 1e-5)
+    assert torch.equal(rd.cpu(), ri)  # the residual sum is exact
+    if dtype == torch.float32:
+        assert (xd.cpu() - xi).abs().max().item() <= 2e-6 * xi.abs().max().item()
+    else:
+        assert ulp_diff16(xd, xi) <= 2
+        assert (xd.cpu() == xi).float().mean().item() > 0.995
+    m = attn.RmsNorm(w.to(device), 1e-5)
+    assert torch.equal(m.forward(x.to(device)), out)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_activations(device, dtype):
+    g = torch.Generator().manual_seed(6)
+    x = (torch.randn((5, 2 * 300), generator=g) * 2).to(dtype)
+    tol = dict(atol=1e-6, rtol=1e-6) if dtype == torch.float32 else None
+    out = torch.empty((5, 300), dtype=dtype, device=device)
+    K.silu_and_mul(out, x.to(device))
+    want = ref.silu_and_mul(x)
+    # expf / tanhf on the GPU and on the CPU may differ in the last place before rounding
+    if tol:
+        assert torch.allclose(out.cpu(), want, **tol)
+    else:
+        assert ulp_diff16(out, want) <= 1
+    for fn, rf in ((K.gelu_new, ref.gelu_new), (K.gelu_fast, ref.gelu_fast)):
+        o = torch.empty_like(x).to(device)
+        fn(o, x.to(device))
+        w = rf(x)
+        if tol:
+            assert torch.allclose(o.cpu(), w, atol=1e-6, rtol=1e-5)
+        else:
+            assert ulp_diff16(o, w) <= 2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_bias_argmax_bias_rows_and_packed_mask(device, dtype):
+    S, V = 9, 128256
+    g = torch.Generator().manual_seed(7)
+    logits = torch.randn((S, V), generator=g).to(dtype)
+    allowed = W.allow_mask(5, S, V, 0.05)
+    allowed[3, :] = False            # nothing allowed: argmax of all -inf is token 0
+    allowed[4, :] = False
+    allowed[4, V - 1] = True         # only the last token
+    packed = np.stack([aici.pack_allowed(a) for a in allowed])
+    rows = np.stack([aici.apply_to_slice_fast(p, aici.bias_row_len(V)) for p in packed])
+    bias = torch.from_numpy(rows)
+    want = aici.biased_argmax(logits, bias)
+    assert want[3].item() == 0 and want[4].item() == V - 1
+    ld = logits.to(device)
+    got_bias, best = K.bias_argmax(ld, bias=bias.to(device), return_logits=True)
+    got_mask = K.bias_argmax(ld, mask=torch.from_numpy(packed).to(device))
+    assert torch.equal(got_bias.cpu().long(), want) and torch.equal(got_mask.cpu().long(), want)
+    picked = logits.float()[torch.arange(S), want]
+    picked[3] = float("-inf")
+    assert torch.equal(best.cpu(), picked)
+    # row indirection: every sequence uses bias row 2
+    sel = torch.full((S,), 2, dtype=torch.int32)
+    got = K.bias_argmax(ld, bias=bias.to(device), bias_rows=sel.to(device))
+    assert torch.equal(got.cpu().long(), aici.biased_argmax(logits, bias[2:3].expand(S, -1)))
+    # ties resolve to the lowest token id
+    flat = torch.zeros((2, 1000), dtype=dtype, device=device)
+    assert K.bias_argmax(flat, bias=torch.zeros((2, 1024), device=device)).tolist() == [0, 0]
+    with pytest.raises(HipAttnError, match="exactly one"):
+        K.bias_argmax(ld)
+
+
+def test_streams_events_and_memory_figures(device):
+    props = K.cuda_get_device_properties(0)
+    assert props.multi_processor_count == 256 and props.total_memory > 200 * 2 ** 30
+    K.cuda_reset_peak_memory_stats(0)
+    st = K.cuda_get_stats_allocated_bytes(0)
+    assert st.current > 0 and st.peak >= st.current
+    assert "GiB" in str(st)
+    s = K.CudaStream()  # pool stream
+    assert s.device_index() == 0 and s.raw != 0 and s.id() == s.raw
+    c = s.clone()
+    assert c.raw == s.raw
+    e0, e1 = K.CudaEvent(timing=True), K.CudaEvent(timing=True)
+    x = torch.ones((1 << 20,), dtype=torch.float16, device=device)
+    out = torch.empty_like(x)
+    torch.cuda.synchronize()  # the pool stream does not order itself after torch's stream
+    import ctypes
+    from aici_amd.kernels import _desc, call
+    e0.record(s)
+    call("hipattn_gelu_new", _desc(out), _desc(x), ctypes.c_void_p(s.raw))  # explicit stream argument
+    e1.record(s)
+    e1.synchronize()
+    assert e0.query() and e1.query() and s.query()
+    assert e0.elapsed_time(e1) >= 0.0
+    s.synchronize()
+    assert torch.allclose(out[:4].float().cpu(), ref.gelu_new(torch.ones(4, dtype=torch.float16)).float())
+    # NULL stream argument = the thread's current stream
+    s.set_current()
+    call("hipattn_gelu_new", _desc(out), _desc(x), None)
+    K.CudaStream.current().synchronize()
+    K.CudaStream.default().set_current()
+    ev = K.CudaEvent()
+    ev.record(K.CudaStream.default())
+    ev.wait(s)
+    s.synchronize()

@@ -131,6 +131,13 @@ def test_sequences_are_independent_and_ragged():
     # empty batch
     e = ref.varlen_attn(q[:0], k[:0], v[:0], cu([]), cu([]), 0, 0, 0.3, True)
     assert e.shape == (0, H, d)
+    # empty sequences inside a batch, and rows without keys, in the fp64 statement
+    lens2 = [4, 0, 3]
+    a = ref.varlen_attn(q[:7], k[:7], v[:7], cu(lens2), cu(lens2), 4, 4, 0.3, True)
+    b = ref.varlen_attn_fp64(q[:7], k[:7], v[:7], cu(lens2), cu(lens2), 0.3, True)
+    assert (a.double() - b).abs().max().item() < 1e-5
+    z = ref.varlen_attn_fp64(q[:5], k[:0], v[:0], cu([5]), cu([0]), 0.3, True)
+    assert torch.all(z == 0)
 
 
 def test_gqa_head_mapping_of_fp64_statement_matches_repeat_kv():
