@@ -25,7 +25,14 @@
 // Numerics follow the reference kernel: fp32 scores and accumulators, softmax
 // in base 2 with scale*log2(e) folded in, un-normalised probabilities rounded
 // to the input dtype as the second product's operand, division by the fp32 sum
-// of the unrounded probabilities at the end.
+// of the unrounded probabilities at the end.  One deliberate difference: the
+// row maximum used as the exponent's reference is only moved when a row
+// outgrows it by more than 2^8, which saves rescaling the accumulators on
+// nearly every tile; probabilities then range up to 256 instead of 1, so the
+// largest one is no longer exactly 1.0 and carries the operand's rounding
+// error (2^-9 relative in bf16, 2^-12 in fp16); the normaliser is given the
+// same rounding for each half-tile's largest term so that it cancels where it
+// matters, on rows that one key dominates.
 #include "common.h"
 #include "device_types.h"
 
@@ -36,6 +43,7 @@ namespace {
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr int BN = 64;  // keys per LDS tile
+constexpr float kRescaleThreshold = 8.0f;  // log2 units: probabilities stay below 256
 
 struct PrefillParams {
   const void *q, *k, *v;
@@ -214,91 +222,102 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
     if (!skip) {
       const T *ks_base = smem + cur * TL::STAGE_ELEMS;
       const T *vs_base = ks_base + TL::K_ELEMS;
+      const bool need_mask = (k0 + BN > Lk) || (p.causal && k0 + BN - 1 > wave_row0 + off);
 
-      // ---- S^T = K . Q^T ------------------------------------------------
-      f32x16_t s[2][QT];
+      // S^T = K . Q^T for the 32 keys of half-tile hf: rows = keys, one query per lane column.
+      auto qk = [&](int hf, f32x16_t(&s)[QT]) {
+        const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kt = 0; kt < 2; kt++)
+        for (int ks = 0; ks < KSTEPS; ks++) {
+          const vec8 a = *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + hf * 32 * TL::KSTR + ks * 16);
 #pragma unroll
-        for (int qt = 0; qt < QT; qt++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) s[kt][qt][i] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ks++) {
-        const vec8 a0 = *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + ks * 16);
-        const vec8 a1 = *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + 32 * TL::KSTR + ks * 16);
+          for (int qt = 0; qt < QT; qt++) s[qt] = Mfma32<T>::run(a, qreg[qt][ks], ks == 0 ? zero : s[qt]);
+        }
+      };
+      // Mask, running maximum with lazy rescaling, exponentials; leaves the B operands of the
+      // second product in pk.  The reference maximum m_ref (log2 domain) only moves when a
+      // row's maximum exceeds it by more than kRescaleThreshold, so probabilities stay below
+      // 2^kRescaleThreshold and the accumulators are rarely touched by the vector ALU.
+      auto softmax = [&](int hf, f32x16_t(&s)[QT], vec8(&pk)[QT][2]) {
 #pragma unroll
         for (int qt = 0; qt < QT; qt++) {
-          s[0][qt] = Mfma32<T>::run(a0, qreg[qt][ks], s[0][qt]);
-          s[1][qt] = Mfma32<T>::run(a1, qreg[qt][ks], s[1][qt]);
-        }
-      }
-
-      // ---- mask + online softmax (one query per lane column) -------------
-      const bool need_mask = (k0 + BN > Lk) || (p.causal && k0 + BN - 1 > wave_row0 + off);
-      vec8 pop[QT][2][2];  // B operands of the second product
-#pragma unroll
-      for (int qt = 0; qt < QT; qt++) {
-        if (need_mask) {
-          const int row = wave_row0 + qt * 32 + c;
-          int limit = p.causal ? row + off : Lk - 1;
-          limit = min(limit, Lk - 1);
-#pragma unroll
-          for (int kt = 0; kt < 2; kt++)
+          if (need_mask) {
+            const int row = wave_row0 + qt * 32 + c;
+            int limit = p.causal ? row + off : Lk - 1;
+            limit = min(limit, Lk - 1);
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-              const int key = k0 + kt * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
-              if (key > limit) s[kt][qt][i] = -INFINITY;
+              const int key = k0 + hf * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
+              if (key > limit) s[qt][i] = -INFINITY;
             }
-        }
-        float mx = -INFINITY;
+          }
+          float mx = s[qt][0];
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++)
+          for (int i = 1; i < 16; i++) mx = fmaxf(mx, s[qt][i]);
+          mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * p.scale_log2;
+          const bool grow = mx > m_run[qt] + kRescaleThreshold;
+          if (__builtin_expect(__any(grow), 0)) {
+            const float m_new = grow ? mx : m_run[qt];
+            // exp2(-inf - finite) = 0 on a row's first keys; rows that do not grow keep 1
+            // (their m_run may still be -inf, and -inf - -inf is not a number).
+            const float alpha = grow ? fast_exp2(m_run[qt] - m_new) : 1.0f;
+            l_run[qt] *= alpha;
 #pragma unroll
-          for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kt][qt][i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run[qt], mx);
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = fast_exp2((m_run[qt] - m_safe) * p.scale_log2);
-        const float msub = m_safe * p.scale_log2;
-        float psum = 0.f;
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++)
+            for (int dt = 0; dt < NDT; dt++) {
+              // Pin the accumulator tile to the accumulation registers at this point, so the
+              // copies the multiply needs are made here, inside the rarely taken branch,
+              // and not hoisted into every iteration.
+              asm volatile("" : "+a"(acc[qt][dt]));
+              acc[qt][dt] *= alpha;
+            }
+            m_run[qt] = m_new;
+          }
+          const float msub = m_run[qt] == -INFINITY ? 0.f : m_run[qt];
+          // The row's largest probability of this half-tile enters the second product
+          // rounded to T; when one key dominates, that rounding is the whole error of the
+          // row.  Put the same rounding into the normaliser (once per row: lane group 0).
+          // It is exactly zero whenever the maximum is the reference itself (p = 1).
+          const float pmax = fast_exp2(mx - msub);
+          float psum = g == 0 ? to_float(from_float<T>(pmax)) - pmax : 0.f;
 #pragma unroll
           for (int half = 0; half < 2; half++) {
-            vec8 pk;
+            vec8 v;
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-              const float e = fast_exp2(s[kt][qt][half * 8 + i] * p.scale_log2 - msub);
+              const float e = fast_exp2(s[qt][half * 8 + i] * p.scale_log2 - msub);
               psum += e;
-              pk[i] = from_float<T>(e);
+              v[i] = from_float<T>(e);
             }
-            pop[qt][kt][half] = pk;
+            pk[qt][half] = v;
           }
-        l_run[qt] = l_run[qt] * alpha + psum;
-        m_run[qt] = m_new;
-        if (__any(alpha != 1.0f)) {
-#pragma unroll
-          for (int dt = 0; dt < NDT; dt++) acc[qt][dt] *= alpha;
+          l_run[qt] += psum;
         }
-      }
-
-      // ---- O^T += V^T . P^T ----------------------------------------------
+      };
+      // O^T += V^T . P^T over the 32 keys of half-tile hf.
+      auto pv = [&](int hf, vec8(&pk)[QT][2]) {
 #pragma unroll
-      for (int dt = 0; dt < NDT; dt++)
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++)
+        for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
           for (int half = 0; half < 2; half++) {
-            const T *vptr = vs_base + v_lane_off + (kt * 32 + half * 16) * TL::VSTR + dt * 32;
+            const T *vptr = vs_base + v_lane_off + (hf * 32 + half * 16) * TL::VSTR + dt * 32;
             const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vptr));
             const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vptr + 8 * TL::VSTR));
             typedef short s16x8 __attribute__((ext_vector_type(8)));
             const s16x8 av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             const vec8 a = bit_cast<vec8>(av);
 #pragma unroll
-            for (int qt = 0; qt < QT; qt++) acc[qt][dt] = Mfma32<T>::run(a, pop[qt][kt][half], acc[qt][dt]);
+            for (int qt = 0; qt < QT; qt++) acc[qt][dt] = Mfma32<T>::run(a, pk[qt][half], acc[qt][dt]);
           }
+      };
+
+      f32x16_t s0[QT], s1[QT];
+      vec8 p0[QT][2], p1[QT][2];
+      qk(0, s0);
+      softmax(0, s0, p0);
+      pv(0, p0);
+      qk(1, s1);
+      softmax(1, s1, p1);
+      pv(1, p1);
     }
     __syncthreads();
   }
@@ -326,7 +345,7 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
     if (p.lse != nullptr && g == 0) {
       // Natural-log sum-exp of the scaled scores; +inf for a row without keys
       // (flash_fwd_kernel.h:629-668).
-      const float lse = l_tot > 0.f ? (m_run[qt] * p.scale_log2 + __builtin_amdgcn_logf(l_tot)) * kLn2 : INFINITY;
+      const float lse = l_tot > 0.f ? (m_run[qt] + __builtin_amdgcn_logf(l_tot)) * kLn2 : INFINITY;
       p.lse[((int64_t)b * p.Hq + h) * p.lse_pitch + row] = lse;
     }
   }

@@ -72,6 +72,9 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (torch copy_) so that FETCH_SIZE / WRITE_SIZE "
+                         "read under rocprofv3 --pmc can be scaled against a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the attention path has no cross-GPU step in this build "
@@ -131,6 +134,15 @@ def main() -> None:
                      "kernel": "paged_decode_kernel (+ reduce) per step, HIP events",
                      "avg_launch_us": round(avg_launch_ms * 1e3, 2)},
     }
+
+    if args.copy_calibration:
+        src = torch.empty((1 << 30,), dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        line["copy_calibration"] = {"bytes_read": 1 << 30, "bytes_written": 1 << 30, "launches": 3}
+        del src, dst
 
     # ---- prefill leg ------------------------------------------------------------------------
     if not args.no_prefill:
