@@ -23,6 +23,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+# HBM bytes per decode launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB
+# copy (profiles/decode_c2_hbm_traffic.md); bench.py cannot read counters itself.
+DECODE_TRAFFIC_BYTES = 641.0e6
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
 
 
@@ -72,6 +75,7 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--kv-pools", type=int, default=3, help="copies of the KV pool cycled through by the decode leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (torch copy_) so that FETCH_SIZE / WRITE_SIZE "
                          "read under rocprofv3 --pmc can be scaled against a kernel of known traffic")
@@ -93,10 +97,18 @@ def main() -> None:
     c_cpu = W.config2()
     c = c_cpu.to(dev)
     out = torch.empty_like(c.q)
+    # Several copies of the KV pool, used round-robin: between two uses of one copy
+    # (pools - 1) x 1.3 GB of other K/V pass through the 256 MB Infinity Cache, so every
+    # step really streams its 634 MB from HBM.
+    pools = [(c.key_cache, c.value_cache)] + [(c.key_cache.clone(), c.value_cache.clone())
+                                              for _ in range(args.kv_pools - 1)]
+    step_no = [0]
 
     def decode_step():
-        K.paged_attention_v1(out, c.q, c.key_cache, c.value_cache, c.num_kv_heads, c.scale, c.block_tables,
-                             c.context_lens, 16, c.max_ctx)
+        kc, vc = pools[step_no[0] % len(pools)]
+        step_no[0] += 1
+        K.paged_attention_v1(out, c.q, kc, vc, c.num_kv_heads, c.scale, c.block_tables, c.context_lens, 16,
+                             c.max_ctx)
 
     for _ in range(args.warmup):
         decode_step()
@@ -128,9 +140,9 @@ def main() -> None:
         "config": {"workload": "paged decode attention: 64 seqs, ctx U[512,4096] (seed 2), 32 q / 8 kv heads, "
                                "d 128, bf16, block 16, tables from a shuffled 20k-block pool",
                    "algorithmic_bytes_per_step": nbytes,
-                   "context_tokens": int(c_cpu.context_lens.sum())},
+                   "context_tokens": int(c_cpu.context_lens.sum()), "kv_pool_copies": len(pools)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": DECODE_TRAFFIC_BYTES,
                      "kernel": "paged_decode_kernel (+ reduce) per step, HIP events",
                      "avg_launch_us": round(avg_launch_ms * 1e3, 2)},
     }
