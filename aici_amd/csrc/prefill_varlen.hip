@@ -351,6 +351,291 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Eight-wavefront variant for head sizes up to 128 and launches large enough
+// to fill the chip.  512 threads own 256 query rows (32 per wavefront) and run
+// two wavefronts per SIMD within 256 registers each: every accumulator lives in
+// a vector register the vector ALU can touch directly, and while one wavefront
+// of a SIMD is in its softmax the other one feeds the matrix pipe.  Eight
+// wavefronts sharing one K/V tile would overload the LDS transpose read
+// (~64 B/clk per CU measured), so this variant stores V transposed instead --
+// V^T[d][key], keys permuted so that the 8 keys a lane needs for one MFMA are
+// contiguous -- and reads both operands with ds_read_b128.
+// ---------------------------------------------------------------------------
+template <int HDP>
+struct TileW8 {
+  static constexpr int KSTR = HDP + 8;   // K rows: key-major, +16 B
+  static constexpr int VTSTR = BN + 8;   // V^T rows: head-element-major, 64 keys + 16 B
+  static constexpr int K_ELEMS = BN * KSTR;
+  static constexpr int V_ELEMS = HDP * VTSTR;
+  static constexpr int STAGE_ELEMS = K_ELEMS + V_ELEMS;
+  static constexpr size_t LDS_BYTES = 2 * (size_t)STAGE_ELEMS * 2;
+};
+
+template <typename T, int HDP>
+__global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams p) {
+  typedef typename Vec8<T>::type vec8;
+  typedef TileW8<HDP> TL;
+  constexpr int KSTEPS = HDP / 16;
+  constexpr int NDT = HDP / 32;
+  constexpr int CPR = HDP / 8;                // 16-byte chunks per K row
+  constexpr int K_CHUNKS = BN * CPR;          // per tile
+  constexpr int NLOADK = (K_CHUNKS + 511) / 512;
+  constexpr int V_ITEMS = 16 * (HDP / 4);     // (4 keys) x (4 head elements) blocks per tile
+  constexpr int NLOADV = (V_ITEMS + 511) / 512;
+  constexpr int BM = 256;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T *smem = reinterpret_cast<T *>(smem_raw);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int g = lane >> 5;
+  const int c = lane & 31;
+
+  int id = blockIdx.x;
+  const int slot = id % p.Hq;
+  id /= p.Hq;
+  const int b = id % p.batch;
+  const int qb = p.n_qblocks - 1 - id / p.batch;
+  const int h = (slot % p.Hkv) * p.G + slot / p.Hkv;
+  const int kvh = h / p.G;
+
+  const int q_begin = p.cu_q[b];
+  const int Lq = p.cu_q[b + 1] - q_begin;
+  const int k_begin = p.cu_k[b];
+  int Lk = p.cu_k[b + 1] - k_begin;
+  if (p.seqused_k) Lk = min(Lk, p.seqused_k[b]);
+  const int wg_row0 = qb * BM;
+  if (wg_row0 >= Lq) return;
+  const int off = Lk - Lq;
+  const int wg_last_row = min(wg_row0 + BM, Lq) - 1;
+  int kmax = p.causal ? min(Lk, wg_last_row + off + 1) : Lk;
+  if (kmax < 0) kmax = 0;
+  const int n_tiles = (kmax + BN - 1) / BN;
+  const int wave_row0 = wg_row0 + wave * 32;
+  const int wave_last_row = wave_row0 + 31;
+
+  const T *qp = static_cast<const T *>(p.q) + (int64_t)q_begin * p.q_row + (int64_t)h * p.q_head;
+  const T *kp = static_cast<const T *>(p.k) + (int64_t)k_begin * p.k_row + (int64_t)kvh * p.k_head;
+  const T *vp = static_cast<const T *>(p.v) + (int64_t)k_begin * p.v_row + (int64_t)kvh * p.v_head;
+  const int d_chunks = p.d / 8;
+
+  vec8 qreg[KSTEPS];
+  {
+    const int row = min(wave_row0 + c, Lq - 1);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      u32x4_t raw = {0u, 0u, 0u, 0u};
+      const int ch = 2 * ks + g;
+      if (ch < d_chunks) raw = *reinterpret_cast<const u32x4_t *>(qp + (int64_t)row * p.q_row + ch * 8);
+      qreg[ks] = bit_cast<vec8>(raw);
+    }
+  }
+  f32x16_t acc[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[dt][i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // ---- tile staging ---------------------------------------------------------
+  // K: chunk (t + 512 i) of the tile, row-major.  V: thread t owns the block of
+  // 4 keys x 4 head elements (kg4, dg); it loads 4 x 8 B, transposes in
+  // registers and writes 4 x 8 B, one per head element, into V^T.  Within a
+  // wavefront 8 lanes cover 8 consecutive dg (64 B of a global row) and 8 lane
+  // groups cover 8 consecutive kg4, which keeps the transposed writes at a
+  // 2-way bank conflict.  Addresses are clamped, never predicated: keys past Lk
+  // re-read the last key (masked later), head elements past d re-read the last
+  // real ones (never stored).
+  u32x4_t kst[NLOADK];
+  u32x2_t vst[NLOADV][4];
+  const int v_dg = (wave & 3) * 8 + (lane & 7);        // + 32 * (item / 512) for HDP > 128 (unused)
+  const int v_kg4 = (wave >> 2) * 8 + (lane >> 3);     // 0..15
+  auto load_tile = [&](int tile) {
+    const int k0 = tile * BN;
+#pragma unroll
+    for (int i = 0; i < NLOADK; i++) {
+      const int idx = min(tid + 512 * i, K_CHUNKS - 1);
+      const int row = idx / CPR, ch = idx % CPR;
+      const int key = min(k0 + row, Lk - 1);
+      kst[i] = *reinterpret_cast<const u32x4_t *>(kp + (int64_t)key * p.k_row + min(ch, d_chunks - 1) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < NLOADV; i++) {
+      const int dg = min(v_dg, p.d / 4 - 1);
+#pragma unroll
+      for (int kk = 0; kk < 4; kk++) {
+        const int key = min(k0 + v_kg4 * 4 + kk, Lk - 1);
+        vst[i][kk] = *reinterpret_cast<const u32x2_t *>(vp + (int64_t)key * p.v_row + dg * 4);
+      }
+    }
+  };
+  auto store_tile = [&](int stage) {
+    T *ks = smem + stage * TL::STAGE_ELEMS;
+    T *vs = ks + TL::K_ELEMS;
+#pragma unroll
+    for (int i = 0; i < NLOADK; i++) {
+      const int idx = tid + 512 * i;
+      if (K_CHUNKS % 512 == 0 || idx < K_CHUNKS) {
+        const int row = idx / CPR, ch = idx % CPR;
+        *reinterpret_cast<u32x4_t *>(ks + row * TL::KSTR + ch * 8) = kst[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NLOADV; i++) {
+      if (V_ITEMS % 512 == 0 || v_dg < HDP / 4) {
+        // 4x4 transpose of 16-bit values: out[dd] = {k0.d, k1.d, k2.d, k3.d}
+        const unsigned a0 = vst[i][0][0], a1 = vst[i][0][1], b0 = vst[i][1][0], b1 = vst[i][1][1];
+        const unsigned c0 = vst[i][2][0], c1 = vst[i][2][1], e0 = vst[i][3][0], e1 = vst[i][3][1];
+        u32x2_t o[4];
+        o[0] = u32x2_t{__builtin_amdgcn_perm(b0, a0, 0x05040100u), __builtin_amdgcn_perm(e0, c0, 0x05040100u)};
+        o[1] = u32x2_t{__builtin_amdgcn_perm(b0, a0, 0x07060302u), __builtin_amdgcn_perm(e0, c0, 0x07060302u)};
+        o[2] = u32x2_t{__builtin_amdgcn_perm(b1, a1, 0x05040100u), __builtin_amdgcn_perm(e1, c1, 0x05040100u)};
+        o[3] = u32x2_t{__builtin_amdgcn_perm(b1, a1, 0x07060302u), __builtin_amdgcn_perm(e1, c1, 0x07060302u)};
+        // Key offset within its group of 16: bits [a(8) g(4) b(2,1)] -> position [g(8) a(4) b].
+        const int o16 = (v_kg4 & 3) * 4;
+        const int pos = (v_kg4 >> 2) * 16 + ((o16 & 4) << 1) + ((o16 & 8) >> 1);
+#pragma unroll
+        for (int dd = 0; dd < 4; dd++)
+          *reinterpret_cast<u32x2_t *>(vs + (v_dg * 4 + dd) * TL::VTSTR + pos) = o[dd];
+      }
+    }
+  };
+
+  if (n_tiles > 0) {
+    load_tile(0);
+    store_tile(0);
+    if (n_tiles > 1) load_tile(1);
+  }
+  __syncthreads();
+
+  const int k_lane_off = c * TL::KSTR + g * 8;
+  const int v_lane_off = c * TL::VTSTR + g * 8;
+
+  for (int j = 0; j < n_tiles; j++) {
+    const int cur = j & 1;
+    if (j + 1 < n_tiles) store_tile(cur ^ 1);
+    if (j + 2 < n_tiles) load_tile(j + 2);
+
+    const int k0 = j * BN;
+    const bool skip = (wave_row0 >= Lq) || (p.causal && k0 > wave_last_row + off);
+    if (!skip) {
+      const T *ks_base = smem + cur * TL::STAGE_ELEMS;
+      const T *vs_base = ks_base + TL::K_ELEMS;
+      const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+      // ---- S^T = K . Q^T for both 32-key halves --------------------------
+      f32x16_t s[2];
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        const vec8 a0 = *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + ks * 16);
+        const vec8 a1 = *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + 32 * TL::KSTR + ks * 16);
+        s[0] = Mfma32<T>::run(a0, qreg[ks], ks == 0 ? zero : s[0]);
+        s[1] = Mfma32<T>::run(a1, qreg[ks], ks == 0 ? zero : s[1]);
+      }
+
+      // ---- mask + online softmax -----------------------------------------
+      const bool need_mask = (k0 + BN > Lk) || (p.causal && k0 + BN - 1 > wave_row0 + off);
+      if (need_mask) {
+        const int row = wave_row0 + c;
+        int limit = p.causal ? row + off : Lk - 1;
+        limit = min(limit, Lk - 1);
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) {
+            const int key = k0 + kt * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
+            if (key > limit) s[kt][i] = -INFINITY;
+          }
+      }
+      float mx = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+      for (int i = 1; i < 16; i++) mx = fmaxf(mx, fmaxf(s[0][i], s[1][i]));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * p.scale_log2;
+      const bool grow = mx > m_run + kRescaleThreshold;
+      if (__builtin_expect(__any(grow), 0)) {
+        const float m_new = grow ? mx : m_run;
+        const float alpha = grow ? fast_exp2(m_run - m_new) : 1.0f;
+        l_run *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) acc[dt] *= alpha;
+        m_run = m_new;
+      }
+      const float msub = m_run == -INFINITY ? 0.f : m_run;
+      const float pmax = fast_exp2(mx - msub);
+      float psum = g == 0 ? to_float(from_float<T>(pmax)) - pmax : 0.f;
+      vec8 pk[2][2];
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+          vec8 v;
+#pragma unroll
+          for (int i = 0; i < 8; i++) {
+            const float e = fast_exp2(s[kt][half * 8 + i] * p.scale_log2 - msub);
+            psum += e;
+            v[i] = from_float<T>(e);
+          }
+          pk[kt][half] = v;
+        }
+      l_run += psum;
+
+      // ---- O^T += V^T . P^T ----------------------------------------------
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+          for (int half = 0; half < 2; half++) {
+            const vec8 a = *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + dt * 32 * TL::VTSTR + kt * 32 + half * 16);
+            acc[dt] = Mfma32<T>::run(a, pk[kt][half], acc[dt]);
+          }
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue ---------------------------------------------------------------
+  T *op = static_cast<T *>(p.out) + (int64_t)q_begin * p.o_row + (int64_t)h * p.o_head;
+  const int row = wave_row0 + c;
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  if (row >= Lq) return;
+  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+#pragma unroll
+  for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+      const int dcol = dt * 32 + a * 8 + g * 4;
+      if (dcol < p.d) {
+        T r[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) r[i] = from_float<T>(acc[dt][a * 4 + i] * inv);
+        *reinterpret_cast<u32x2_t *>(op + (int64_t)row * p.o_row + dcol) = *reinterpret_cast<u32x2_t *>(r);
+      }
+    }
+  if (p.lse != nullptr && g == 0) {
+    const float lse = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : INFINITY;
+    p.lse[((int64_t)b * p.Hq + h) * p.lse_pitch + row] = lse;
+  }
+}
+
+template <typename T, int HDP>
+void launch_prefill_w8(PrefillParams p, hipStream_t stream) {
+  static bool attr_set = false;  // benign race: setting twice is harmless
+  auto kernel = prefill_varlen_w8_kernel<T, HDP>;
+  if (!attr_set) {
+    HA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)TileW8<HDP>::LDS_BYTES));
+    attr_set = true;
+  }
+  p.n_qblocks = (p.max_q + 255) / 256;
+  const int64_t n_wg = (int64_t)p.n_qblocks * p.batch * p.Hq;
+  HA_CHECK(n_wg <= 0x7fffffff, "mha_varlen_fwd: too many workgroups");
+  kernel<<<dim3((unsigned)n_wg), 512, TileW8<HDP>::LDS_BYTES, stream>>>(p);
+  check_launch("mha_varlen_fwd");
+}
+
 template <typename T, int HDP, int QT>
 void launch_prefill(PrefillParams p, hipStream_t stream) {
   constexpr int BM = 4 * QT * 32;
@@ -374,7 +659,13 @@ void pick_qt(const PrefillParams &p, int64_t total_q, hipStream_t stream) {
   // fill the 256 CUs; small launches use 128-row workgroups.
   if constexpr (HDP <= 128) {
     const int64_t wg256 = (total_q / 256 + p.batch) * p.Hq;
-    if (wg256 >= 2 * 256) {
+    const char *force = getenv("HIPATTN_PREFILL_KERNEL");  // tuning aid: "w8", "qt2" or "qt1"
+    const bool big = wg256 >= 2 * 256;
+    if (force ? !strcmp(force, "w8") : big) {
+      launch_prefill_w8<T, HDP>(p, stream);
+      return;
+    }
+    if (force ? !strcmp(force, "qt2") : false) {
       launch_prefill<T, HDP, 2>(p, stream);
       return;
     }
