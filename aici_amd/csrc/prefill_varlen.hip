@@ -76,6 +76,14 @@ struct Mfma32<bf16_t> {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// max(a, b, c) in one instruction.  Scores are never NaN here, so the
+// canonicalising copies fmaxf would add to every MFMA result are not needed.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 // Row strides of the LDS tiles in elements.  K is read as 16 B per lane with
 // 16 consecutive rows per access phase, V as 64 B runs of 4 consecutive rows;
 // the paddings make those phases hit distinct banks.
@@ -369,7 +377,7 @@ struct TileW8 {
   static constexpr int K_ELEMS = BN * KSTR;
   static constexpr int V_ELEMS = HDP * VTSTR;
   static constexpr int STAGE_ELEMS = K_ELEMS + V_ELEMS;
-  static constexpr size_t LDS_BYTES = 2 * (size_t)STAGE_ELEMS * 2;
+  static constexpr size_t LDS_BYTES = 3 * (size_t)STAGE_ELEMS * 2;
 };
 
 template <typename T, int HDP>
@@ -383,6 +391,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   constexpr int NLOADK = (K_CHUNKS + 511) / 512;
   constexpr int V_ITEMS = 16 * (HDP / 4);     // (4 keys) x (4 head elements) blocks per tile
   constexpr int NLOADV = (V_ITEMS + 511) / 512;
+  static_assert(NLOADV == 1, "one (4 keys x 4 elements) block per thread");
   constexpr int BM = 256;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -451,24 +460,38 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   // real ones (never stored).
   u32x4_t kst[NLOADK];
   u32x2_t vst[NLOADV][4];
-  const int v_dg = (wave & 3) * 8 + (lane & 7);        // + 32 * (item / 512) for HDP > 128 (unused)
-  const int v_kg4 = (wave >> 2) * 8 + (lane >> 3);     // 0..15
+  const int v_dg = (wave & 3) * 8 + (lane & 7);        // 4-element group of the head dimension
+  const int v_kg4 = (wave >> 2) * 8 + (lane >> 3);     // 4-key group of the tile, 0..15
+  // Per-thread element offsets inside a tile, relative to its first key; a
+  // full tile only adds the tile's base (one 64-bit add per load).
+  int64_t k_toff[NLOADK], v_toff[4];
+#pragma unroll
+  for (int i = 0; i < NLOADK; i++) {
+    const int idx = min(tid + 512 * i, K_CHUNKS - 1);
+    k_toff[i] = (int64_t)(idx / CPR) * p.k_row + min(idx % CPR, d_chunks - 1) * 8;
+  }
+#pragma unroll
+  for (int kk = 0; kk < 4; kk++) v_toff[kk] = (int64_t)(v_kg4 * 4 + kk) * p.v_row + min(v_dg, p.d / 4 - 1) * 4;
   auto load_tile = [&](int tile) {
     const int k0 = tile * BN;
+    if (k0 + BN <= Lk) {
+      const T *kt = kp + (int64_t)k0 * p.k_row;
+      const T *vt = vp + (int64_t)k0 * p.v_row;
 #pragma unroll
-    for (int i = 0; i < NLOADK; i++) {
-      const int idx = min(tid + 512 * i, K_CHUNKS - 1);
-      const int row = idx / CPR, ch = idx % CPR;
-      const int key = min(k0 + row, Lk - 1);
-      kst[i] = *reinterpret_cast<const u32x4_t *>(kp + (int64_t)key * p.k_row + min(ch, d_chunks - 1) * 8);
-    }
+      for (int i = 0; i < NLOADK; i++) kst[i] = *reinterpret_cast<const u32x4_t *>(kt + k_toff[i]);
 #pragma unroll
-    for (int i = 0; i < NLOADV; i++) {
-      const int dg = min(v_dg, p.d / 4 - 1);
+      for (int kk = 0; kk < 4; kk++) vst[0][kk] = *reinterpret_cast<const u32x2_t *>(vt + v_toff[kk]);
+    } else {  // the last, partial tile: clamp every key to the last real one
+#pragma unroll
+      for (int i = 0; i < NLOADK; i++) {
+        const int idx = min(tid + 512 * i, K_CHUNKS - 1);
+        const int key = min(k0 + idx / CPR, Lk - 1);
+        kst[i] = *reinterpret_cast<const u32x4_t *>(kp + (int64_t)key * p.k_row + min(idx % CPR, d_chunks - 1) * 8);
+      }
 #pragma unroll
       for (int kk = 0; kk < 4; kk++) {
         const int key = min(k0 + v_kg4 * 4 + kk, Lk - 1);
-        vst[i][kk] = *reinterpret_cast<const u32x2_t *>(vp + (int64_t)key * p.v_row + dg * 4);
+        vst[0][kk] = *reinterpret_cast<const u32x2_t *>(vp + (int64_t)key * p.v_row + min(v_dg, p.d / 4 - 1) * 4);
       }
     }
   };
@@ -513,87 +536,138 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
 
   const int k_lane_off = c * TL::KSTR + g * 8;
   const int v_lane_off = c * TL::VTSTR + g * 8;
+  const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  for (int j = 0; j < n_tiles; j++) {
-    const int cur = j & 1;
-    if (j + 1 < n_tiles) store_tile(cur ^ 1);
-    if (j + 2 < n_tiles) load_tile(j + 2);
-
-    const int k0 = j * BN;
-    const bool skip = (wave_row0 >= Lq) || (p.causal && k0 > wave_last_row + off);
-    if (!skip) {
-      const T *ks_base = smem + cur * TL::STAGE_ELEMS;
-      const T *vs_base = ks_base + TL::K_ELEMS;
-      const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-
-      // ---- S^T = K . Q^T for both 32-key halves --------------------------
-      f32x16_t s[2];
+  // ---- the three phases of one 64-key tile ------------------------------------
+  // Q: S^T = K . Q^T for both 32-key halves; LDS reads run two contraction
+  // steps ahead of the MFMAs that consume them.
+  auto phase_qk = [&](int buf, f32x16_t(&s)[2]) {
+    const T *ks_base = smem + buf * TL::STAGE_ELEMS;
+    auto rd = [&](int kt, int ks) -> vec8 {
+      return *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + kt * 32 * TL::KSTR + ks * 16);
+    };
+    vec8 ka[3][2];
+    ka[0][0] = rd(0, 0);
+    ka[0][1] = rd(1, 0);
+    if (KSTEPS > 1) {
+      ka[1][0] = rd(0, 1);
+      ka[1][1] = rd(1, 1);
+    }
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ks++) {
-        const vec8 a0 = *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + ks * 16);
-        const vec8 a1 = *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + 32 * TL::KSTR + ks * 16);
-        s[0] = Mfma32<T>::run(a0, qreg[ks], ks == 0 ? zero : s[0]);
-        s[1] = Mfma32<T>::run(a1, qreg[ks], ks == 0 ? zero : s[1]);
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      if (ks + 2 < KSTEPS) {
+        ka[(ks + 2) % 3][0] = rd(0, ks + 2);
+        ka[(ks + 2) % 3][1] = rd(1, ks + 2);
       }
-
-      // ---- mask + online softmax -----------------------------------------
-      const bool need_mask = (k0 + BN > Lk) || (p.causal && k0 + BN - 1 > wave_row0 + off);
-      if (need_mask) {
-        const int row = wave_row0 + c;
-        int limit = p.causal ? row + off : Lk - 1;
-        limit = min(limit, Lk - 1);
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const int key = k0 + kt * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
-            if (key > limit) s[kt][i] = -INFINITY;
-          }
-      }
-      float mx = fmaxf(s[0][0], s[1][0]);
-#pragma unroll
-      for (int i = 1; i < 16; i++) mx = fmaxf(mx, fmaxf(s[0][i], s[1][i]));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * p.scale_log2;
-      const bool grow = mx > m_run + kRescaleThreshold;
-      if (__builtin_expect(__any(grow), 0)) {
-        const float m_new = grow ? mx : m_run;
-        const float alpha = grow ? fast_exp2(m_run - m_new) : 1.0f;
-        l_run *= alpha;
-#pragma unroll
-        for (int dt = 0; dt < NDT; dt++) acc[dt] *= alpha;
-        m_run = m_new;
-      }
-      const float msub = m_run == -INFINITY ? 0.f : m_run;
-      const float pmax = fast_exp2(mx - msub);
-      float psum = g == 0 ? to_float(from_float<T>(pmax)) - pmax : 0.f;
-      vec8 pk[2][2];
+      __builtin_amdgcn_sched_barrier(0);
+      s[0] = Mfma32<T>::run(ka[ks % 3][0], qreg[ks], ks == 0 ? zero : s[0]);
+      s[1] = Mfma32<T>::run(ka[ks % 3][1], qreg[ks], ks == 0 ? zero : s[1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // S: mask, running maximum (moved lazily), exponentials -> MFMA operands.
+  auto phase_softmax = [&](int k0, f32x16_t(&s)[2], vec8(&pk)[2][2]) {
+    const bool need_mask = (k0 + BN > Lk) || (p.causal && k0 + BN - 1 > wave_row0 + off);
+    if (need_mask) {
+      const int row = wave_row0 + c;
+      int limit = p.causal ? row + off : Lk - 1;
+      limit = min(limit, Lk - 1);
 #pragma unroll
       for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-        for (int half = 0; half < 2; half++) {
-          vec8 v;
-#pragma unroll
-          for (int i = 0; i < 8; i++) {
-            const float e = fast_exp2(s[kt][half * 8 + i] * p.scale_log2 - msub);
-            psum += e;
-            v[i] = from_float<T>(e);
-          }
-          pk[kt][half] = v;
+        for (int i = 0; i < 16; i++) {
+          const int key = k0 + kt * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
+          if (key > limit) s[kt][i] = -INFINITY;
         }
-      l_run += psum;
-
-      // ---- O^T += V^T . P^T ----------------------------------------------
-#pragma unroll
-      for (int dt = 0; dt < NDT; dt++)
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-          for (int half = 0; half < 2; half++) {
-            const vec8 a = *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + dt * 32 * TL::VTSTR + kt * 32 + half * 16);
-            acc[dt] = Mfma32<T>::run(a, pk[kt][half], acc[dt]);
-          }
     }
-    __syncthreads();
+    float mx = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+    for (int i = 1; i < 16; i++) mx = max3(mx, s[0][i], s[1][i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * p.scale_log2;
+    const bool grow = mx > m_run + kRescaleThreshold;
+    if (__builtin_expect(__any(grow), 0)) {
+      const float m_new = grow ? mx : m_run;
+      const float alpha = grow ? fast_exp2(m_run - m_new) : 1.0f;
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++) acc[dt] *= alpha;
+      m_run = m_new;
+    }
+    const float msub = m_run == -INFINITY ? 0.f : m_run;
+    const float pmax = fast_exp2(mx - msub);
+    float psum = g == 0 ? to_float(from_float<T>(pmax)) - pmax : 0.f;
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int half = 0; half < 2; half++) {
+        vec8 v;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          const float e = fast_exp2(s[kt][half * 8 + i] * p.scale_log2 - msub);
+          psum += e;
+          v[i] = from_float<T>(e);
+        }
+        pk[kt][half] = v;
+      }
+    l_run += psum;
+  };
+  // P: O^T += V^T . P^T; step n = (dt, kt, half), its operand is read four steps ahead.
+  auto phase_pv = [&](int buf, vec8(&pk)[2][2]) {
+    const T *vs_base = smem + buf * TL::STAGE_ELEMS + TL::K_ELEMS;
+    constexpr int NSTEP = NDT * 4;
+    auto rd = [&](int n) -> vec8 {
+      const int dt = n / 4, kt = (n / 2) % 2, half = n % 2;
+      return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + dt * 32 * TL::VTSTR + kt * 32 + half * 16);
+    };
+    vec8 va[5];
+#pragma unroll
+    for (int n = 0; n < 4 && n < NSTEP; n++) va[n] = rd(n);
+#pragma unroll
+    for (int n = 0; n < NSTEP; n++) {
+      if (n + 4 < NSTEP) va[(n + 4) % 5] = rd(n + 4);
+      __builtin_amdgcn_sched_barrier(0);
+      acc[n / 4] = Mfma32<T>::run(va[n % 5], pk[(n / 2) % 2][n % 2], acc[n / 4]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // Tiles entirely past the diagonal of every row of this wavefront are skipped.
+  auto skip_tile = [&](int j) { return (wave_row0 >= Lq) || (p.causal && j * BN > wave_last_row + off); };
+
+  // The two wavefronts that share a SIMD run the phases in different orders
+  // between two workgroup barriers -- wavefronts 0-3: Q S P of tile j;
+  // wavefronts 4-7: P of tile j-1, then Q S of tile j -- so that one is on the
+  // vector ALU while the other is on the matrix pipe instead of both queueing
+  // for the same unit.  V of tile j-1 must therefore survive iteration j:
+  // three tile buffers.
+  if (wave < 4) {
+    for (int j = 0; j < n_tiles; j++) {
+      if (j + 1 < n_tiles) store_tile((j + 1) % 3);
+      if (j + 2 < n_tiles) load_tile(j + 2);
+      if (!skip_tile(j)) {
+        f32x16_t s[2];
+        vec8 pk[2][2];
+        phase_qk(j % 3, s);
+        phase_softmax(j * BN, s, pk);
+        phase_pv(j % 3, pk);
+      }
+      __syncthreads();
+    }
+  } else {
+    vec8 pk[2][2];
+    bool pending = false;
+    for (int j = 0; j < n_tiles; j++) {
+      if (j + 1 < n_tiles) store_tile((j + 1) % 3);
+      if (j + 2 < n_tiles) load_tile(j + 2);
+      if (pending) phase_pv((j + 2) % 3, pk);  // tile j-1
+      pending = !skip_tile(j);
+      if (pending) {
+        f32x16_t s[2];
+        phase_qk(j % 3, s);
+        phase_softmax(j * BN, s, pk);
+      }
+      __syncthreads();
+    }
+    if (pending) phase_pv((n_tiles + 2) % 3, pk);  // tile n_tiles-1
   }
 
   // ---- epilogue ---------------------------------------------------------------
