@@ -60,6 +60,10 @@ struct DecodeParams {
   void *tmp_out;  // [S, Hq, P, HD] in T (reference v2 format)
   void *out;      // [S, Hq, HD]
   int64_t out_stride;
+  // flat split (paged_decode_flat_kernel)
+  int *flat_prefix;  // [S + 1] block pairs before each sequence, written by workgroup 0
+  int flat_waves;    // wavefronts of the main launch
+  int flat_cols;     // query-head columns kept per partial slot: min(G, 16)
 };
 
 template <typename T>
@@ -78,6 +82,141 @@ struct Mfma16<bf16_t> {
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// The cache bytes of one block pair of one kv head, as MFMA operands.
+template <int HD>
+struct PairRegs {
+  u32x4_t kra[(HD + 31) / 32], krb[(HD + 31) / 32];
+  u32x2_t vra[HD / 16], vrb[HD / 16];
+};
+
+// Issues the loads of the block pair (pa, pb) of one kv head.
+template <typename T, int HD>
+__device__ __forceinline__ void pair_load(const DecodeParams &p, const T *kbase, const T *vbase, int64_t pa, int64_t pb,
+                                          PairRegs<HD> &r) {
+  constexpr int NCH = HD / 8;
+  constexpr int NSTEP = (HD + 31) / 32;
+  constexpr int NDT = HD / 16;
+  const int lane = threadIdx.x & 63;
+  const int kg = lane >> 4;
+  const int col = lane & 15;
+  const int64_t last_block = p.num_blocks - 1;
+  pa = pa < 0 ? 0 : (pa > last_block ? last_block : pa);
+  pb = pb < 0 ? 0 : (pb > last_block ? last_block : pb);
+  const T *ka = kbase + pa * p.k_block_stride;
+  const T *kb = kbase + pb * p.k_block_stride;
+  const T *va = vbase + pa * p.v_block_stride;
+  const T *vb = vbase + pb * p.v_block_stride;
+  // K: step s of a block is the contiguous 1 KiB run of chunks 4s..4s+3.
+#pragma unroll
+  for (int s = 0; s < NSTEP; s++) {
+    const int ch = 4 * s + kg;
+    r.kra[s] = u32x4_t{0u, 0u, 0u, 0u};
+    r.krb[s] = u32x4_t{0u, 0u, 0u, 0u};
+    if (NCH % 4 == 0 || ch < NCH) {
+      r.kra[s] = *reinterpret_cast<const u32x4_t *>(ka + (ch * kBlockSize + col) * 8);
+      r.krb[s] = *reinterpret_cast<const u32x4_t *>(kb + (ch * kBlockSize + col) * 8);
+    }
+  }
+  // V: tile dt of a block is the contiguous 512 B run of rows 16dt..16dt+15;
+  // lane (kg, row) takes tokens 4kg..4kg+3 of its row.
+#pragma unroll
+  for (int dt = 0; dt < NDT; dt++) {
+    r.vra[dt] = *reinterpret_cast<const u32x2_t *>(va + (dt * 16 + col) * kBlockSize + kg * 4);
+    r.vrb[dt] = *reinterpret_cast<const u32x2_t *>(vb + (dt * 16 + col) * kBlockSize + kg * 4);
+  }
+}
+
+// Folds a loaded block pair -- blocks `blk` and `blk + 1` of the context, the
+// second absent when !has_b -- into the running softmax state (m_run, l_run,
+// acc).  qreg: lane (kg, col) holds q[head col][32*step + 8*kg .. +8].
+template <typename T, int HD>
+__device__ __forceinline__ void pair_compute(const DecodeParams &p, PairRegs<HD> &r, int blk, bool has_b, int ctx,
+                                             float slope, const typename Vec8<T>::type (&qreg)[(HD + 31) / 32],
+                                             float &m_run, float &l_run, f32x4_t (&acc)[HD / 16]) {
+  typedef typename Vec8<T>::type vec8;
+  constexpr int NSTEP = (HD + 31) / 32;
+  constexpr int NDT = HD / 16;
+  const int lane = threadIdx.x & 63;
+  const int kg = lane >> 4;
+  u32x4_t(&kra)[NSTEP] = r.kra;
+  u32x4_t(&krb)[NSTEP] = r.krb;
+  u32x2_t(&vra)[NDT] = r.vra;
+  u32x2_t(&vrb)[NDT] = r.vrb;
+
+  // S^T = K . Q^T : rows = tokens of the block, columns = query heads.
+  f32x4_t sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < NSTEP; s++) {
+    sa = Mfma16<T>::run(bit_cast<vec8>(kra[s]), qreg[s], sa);
+    sb = Mfma16<T>::run(bit_cast<vec8>(krb[s]), qreg[s], sb);
+  }
+
+  // Lane (kg, col) now holds tokens 4kg..4kg+3 of both blocks for head col.
+  const int tok_a = blk * kBlockSize + kg * 4;
+  const int tok_b = has_b ? tok_a + kBlockSize : 0x3fffffff;
+  float x[8];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    x[i] = sa[i] * p.scale_log2 + slope * (float)(tok_a + i - ctx + 1);
+    x[4 + i] = sb[i] * p.scale_log2 + slope * (float)(tok_b + i - ctx + 1);
+    if (tok_a + i >= ctx) x[i] = -INFINITY;
+    if (tok_b + i >= ctx) x[4 + i] = -INFINITY;
+  }
+  float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  const float m_new = fmaxf(m_run, mx);
+  const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+  const float alpha = fast_exp2(m_run - m_safe);
+  float psum = 0.f;
+  vec8 pv;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const float e = fast_exp2(x[i] - m_safe);
+    psum += e;
+    pv[i] = from_float<T>(e);
+  }
+  l_run = l_run * alpha + psum;
+  m_run = m_new;
+  if (__any(alpha != 1.0f)) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++) acc[dt] *= alpha;
+  }
+
+  // Tokens past the context hold whatever the cache held before; a zero
+  // probability does not neutralise a NaN, so clear those V entries.
+  if ((blk + 2) * kBlockSize > ctx || !has_b) {  // wave-uniform: only the context's last pair
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++) {
+      uint16_t *ea = reinterpret_cast<uint16_t *>(&vra[dt]);
+      uint16_t *eb = reinterpret_cast<uint16_t *>(&vrb[dt]);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        if (tok_a + i >= ctx) ea[i] = 0;
+        if (tok_b + i >= ctx) eb[i] = 0;
+      }
+    }
+  }
+
+  // O^T += V^T . P^T : contraction slot 8kg+j is token 4kg+j of block A
+  // (j < 4) or token 4kg+j-4 of block B.
+#pragma unroll
+  for (int dt = 0; dt < NDT; dt++) {
+    u32x4_t a = {vra[dt][0], vra[dt][1], vrb[dt][0], vrb[dt][1]};
+    acc[dt] = Mfma16<T>::run(bit_cast<vec8>(a), pv, acc[dt]);
+  }
+}
+
+template <typename T, int HD>
+__device__ __forceinline__ void pair_step(const DecodeParams &p, const T *kbase, const T *vbase, int64_t pa, int64_t pb,
+                                          int blk, bool has_b, int ctx, float slope,
+                                          const typename Vec8<T>::type (&qreg)[(HD + 31) / 32], float &m_run,
+                                          float &l_run, f32x4_t (&acc)[HD / 16]) {
+  PairRegs<HD> r;
+  pair_load<T, HD>(p, kbase, vbase, pa, pb, r);
+  pair_compute<T, HD>(p, r, blk, has_b, ctx, slope, qreg, m_run, l_run, acc);
+}
 
 // V2FMT: write partials in the reference's v2 layout (normalised T outputs,
 // natural-log maxima) instead of the internal fp32 one.
@@ -141,8 +280,6 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(DecodeParams p) {
   }
   const float slope = (p.alibi != nullptr && col_ok) ? p.alibi[qh] * kLog2e : 0.f;
 
-  const int64_t last_block = p.num_blocks - 1;
-
   const T *kbase = static_cast<const T *>(p.kc) + (int64_t)kvh * p.k_head_stride;
   const T *vbase = static_cast<const T *>(p.vc) + (int64_t)kvh * p.v_head_stride;
 
@@ -154,98 +291,9 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(DecodeParams p) {
 
   for (int it = 2 * wave; it < nb; it += 8) {
     const bool has_b = it + 1 < nb;
-    int64_t pa = __builtin_amdgcn_readlane(tbl, it);
-    int64_t pb = __builtin_amdgcn_readlane(tbl, has_b ? it + 1 : it);
-    pa = pa < 0 ? 0 : (pa > last_block ? last_block : pa);
-    pb = pb < 0 ? 0 : (pb > last_block ? last_block : pb);
-    const T *ka = kbase + pa * p.k_block_stride;
-    const T *kb = kbase + pb * p.k_block_stride;
-    const T *va = vbase + pa * p.v_block_stride;
-    const T *vb = vbase + pb * p.v_block_stride;
-
-    // K: step s of a block is the contiguous 1 KiB run of chunks 4s..4s+3.
-    u32x4_t kra[NSTEP], krb[NSTEP];
-#pragma unroll
-    for (int s = 0; s < NSTEP; s++) {
-      const int ch = 4 * s + kg;
-      kra[s] = u32x4_t{0u, 0u, 0u, 0u};
-      krb[s] = u32x4_t{0u, 0u, 0u, 0u};
-      if (NCH % 4 == 0 || ch < NCH) {
-        kra[s] = *reinterpret_cast<const u32x4_t *>(ka + (ch * kBlockSize + col) * 8);
-        krb[s] = *reinterpret_cast<const u32x4_t *>(kb + (ch * kBlockSize + col) * 8);
-      }
-    }
-    // V: tile dt of a block is the contiguous 512 B run of rows 16dt..16dt+15;
-    // lane (kg, row) takes tokens 4kg..4kg+3 of its row.
-    u32x2_t vra[NDT], vrb[NDT];
-#pragma unroll
-    for (int dt = 0; dt < NDT; dt++) {
-      vra[dt] = *reinterpret_cast<const u32x2_t *>(va + (dt * 16 + col) * kBlockSize + kg * 4);
-      vrb[dt] = *reinterpret_cast<const u32x2_t *>(vb + (dt * 16 + col) * kBlockSize + kg * 4);
-    }
-
-    // S^T = K . Q^T : rows = tokens of the block, columns = query heads.
-    f32x4_t sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < NSTEP; s++) {
-      sa = Mfma16<T>::run(bit_cast<vec8>(kra[s]), qreg[s], sa);
-      sb = Mfma16<T>::run(bit_cast<vec8>(krb[s]), qreg[s], sb);
-    }
-
-    // Lane (kg, col) now holds tokens 4kg..4kg+3 of both blocks for head col.
-    const int tok_a = (b0 + it) * kBlockSize + kg * 4;
-    const int tok_b = has_b ? tok_a + kBlockSize : 0x3fffffff;
-    float x[8];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      x[i] = sa[i] * p.scale_log2 + slope * (float)(tok_a + i - ctx + 1);
-      x[4 + i] = sb[i] * p.scale_log2 + slope * (float)(tok_b + i - ctx + 1);
-      if (tok_a + i >= ctx) x[i] = -INFINITY;
-      if (tok_b + i >= ctx) x[4 + i] = -INFINITY;
-    }
-    float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run, mx);
-    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = fast_exp2(m_run - m_safe);
-    float psum = 0.f;
-    vec8 pv;
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const float e = fast_exp2(x[i] - m_safe);
-      psum += e;
-      pv[i] = from_float<T>(e);
-    }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    if (__any(alpha != 1.0f)) {
-#pragma unroll
-      for (int dt = 0; dt < NDT; dt++) acc[dt] *= alpha;
-    }
-
-    // Tokens past the context hold whatever the cache held before; a zero
-    // probability does not neutralise a NaN, so clear those V entries.
-    if ((b0 + it + 2) * kBlockSize > ctx || !has_b) {  // wave-uniform: only the context's last pair
-#pragma unroll
-      for (int dt = 0; dt < NDT; dt++) {
-        uint16_t *ea = reinterpret_cast<uint16_t *>(&vra[dt]);
-        uint16_t *eb = reinterpret_cast<uint16_t *>(&vrb[dt]);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          if (tok_a + i >= ctx) ea[i] = 0;
-          if (tok_b + i >= ctx) eb[i] = 0;
-        }
-      }
-    }
-
-    // O^T += V^T . P^T : contraction slot 8kg+j is token 4kg+j of block A
-    // (j < 4) or token 4kg+j-4 of block B.
-#pragma unroll
-    for (int dt = 0; dt < NDT; dt++) {
-      u32x4_t a = {vra[dt][0], vra[dt][1], vrb[dt][0], vrb[dt][1]};
-      acc[dt] = Mfma16<T>::run(bit_cast<vec8>(a), pv, acc[dt]);
-    }
+    const int64_t pa = __builtin_amdgcn_readlane(tbl, it);
+    const int64_t pb = __builtin_amdgcn_readlane(tbl, has_b ? it + 1 : it);
+    pair_step<T, HD>(p, kbase, vbase, pa, pb, b0 + it, has_b, ctx, slope, qreg, m_run, l_run, acc);
   }
 
   float l_tot = l_run + __shfl_xor(l_run, 16, 64);
@@ -372,6 +420,340 @@ void dispatch_head(const DecodeParams &p, int head_size, int64_t S, hipStream_t 
     case 256: launch_decode<T, 256, V2FMT>(p, S, stream); break;
     default: fail("paged_attention: unsupported head size %d (supported: 64, 80, 96, 112, 128, 256)", head_size);
   }
+}
+
+// ---------------------------------------------------------------------------
+// Flat split.  The launch above hands out (sequence, kv head, partition) items
+// of unequal length, and every workgroup pays a chain of dependent loads
+// (context length -> table -> cache) before its first byte streams.  Here the
+// whole step is one list of units -- a unit is one block pair of one
+// (sequence, kv head) segment, ordered sequence-major with the pair fastest --
+// and the list is cut into equal contiguous ranges, one per wavefront of a
+// launch sized to what the chip holds at once.  Every wavefront therefore
+// streams the same number of bytes, starts once, and the launch drains
+// together.  A range may begin inside a segment and end inside a later one, so
+// a wavefront emits at most two partial results (slot 2w: the piece that
+// begins where its range begins; slot 2w+1: a later piece cut by the range's
+// end); segments that lie inside one range are normalised and written to
+// `out` directly.  The reduce kernel recomputes which wavefronts cover a
+// segment from the same arithmetic.
+// ---------------------------------------------------------------------------
+constexpr int kFlatMaxSeqs = 1024;
+
+__device__ __forceinline__ int ctx_pairs(int ctx) {
+  return ctx > 0 ? (ctx + 2 * kBlockSize - 1) / (2 * kBlockSize) : 0;
+}
+
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// `units` cut into `waves` contiguous ranges whose lengths differ by at most
+// one (the first `rem` ranges hold `base + 1` units).
+struct FlatSplit {
+  int base, rem;
+  __device__ FlatSplit(int units, int waves) : base(units / waves), rem(units % waves) {}
+  __device__ int start(int w) const { return w * base + min(w, rem); }
+  __device__ int wave_of(int u) const {
+    const int split = rem * (base + 1);
+    return u < split ? u / (base + 1) : rem + (u - split) / base;
+  }
+};
+
+template <typename T, int HD>
+__global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void paged_decode_flat_kernel(DecodeParams p) {
+  typedef typename Vec8<T>::type vec8;
+  constexpr int NCH = HD / 8;
+  constexpr int NSTEP = (HD + 31) / 32;
+  constexpr int NDT = HD / 16;
+  __shared__ int s_ctx[kFlatMaxSeqs];
+  __shared__ int s_excl[kFlatMaxSeqs + 1];  // block pairs before sequence s; [S] = all
+  __shared__ int s_wsum[4];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int kg = lane >> 4;
+  const int col = lane & 15;
+  const int S = p.num_seqs;
+
+  // Exclusive prefix of the pair counts, thread t owning sequences 4t..4t+3.
+  {
+    int c[4], n[4], tsum = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int s = 4 * tid + j;
+      c[j] = s < S ? p.context_lens[s] : 0;
+      n[j] = ctx_pairs(c[j]);
+      tsum += n[j];
+    }
+    int inc = tsum;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(inc, o, 64);
+      if (lane >= o) inc += t;
+    }
+    if (lane == 63) s_wsum[wave] = inc;
+    __syncthreads();
+    int run = inc - tsum;
+    for (int k = 0; k < wave; k++) run += s_wsum[k];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int s = 4 * tid + j;
+      if (s < S) {
+        s_ctx[s] = c[j];
+        s_excl[s] = run;
+      }
+      run += n[j];
+    }
+    if (tid == 0) s_excl[S] = s_wsum[0] + s_wsum[1] + s_wsum[2] + s_wsum[3];
+    __syncthreads();
+  }
+  if (blockIdx.x == 0) {
+    for (int s = tid; s <= S; s += 256) p.flat_prefix[s] = s_excl[s];
+  }
+
+  const int hk = p.Hkv * p.col_groups;
+  const int total_units = hk * uniform(s_excl[S]);  // the host bounds this below 2^31
+  const FlatSplit split(total_units, p.flat_waves);
+  const int w = blockIdx.x * 4 + wave;
+  const int u_first = split.start(w);
+  const int u_end = split.start(w + 1);
+  if (u_first >= u_end) return;
+
+  // The sequence holding unit u_first: the first s with hk * pairs_before(s + 1) > u_first.
+  int seq = 0;
+  for (int s0 = 0; s0 < S; s0 += 64) {
+    const int s = s0 + lane;
+    const bool past = s < S && hk * s_excl[s + 1] > u_first;
+    const unsigned long long b = __ballot(past);
+    if (b) {
+      seq = s0 + __ffsll(b) - 1;
+      break;
+    }
+  }
+
+  T *out = static_cast<T *>(p.out);
+  int u = u_first;
+  while (u < u_end) {
+    const int before = uniform(s_excl[seq]);
+    const int pairs = uniform(s_excl[seq + 1]) - before;
+    if (pairs == 0) {  // u < total_units, so a longer sequence follows
+      seq++;
+      continue;
+    }
+    const int ctx = uniform(s_ctx[seq]);
+    const int nblk = (ctx + kBlockSize - 1) / kBlockSize;
+    const int r = u - hk * before;
+    const int h = r / pairs;
+    const int pr0 = r - h * pairs;
+    const int n = min(pairs - pr0, u_end - u);
+    const int kvh = h / p.col_groups;
+    const int cg = h - kvh * p.col_groups;
+    const int g_idx = cg * 16 + col;
+    const bool col_ok = g_idx < p.G;
+    const int qh = kvh * p.G + g_idx;
+
+    vec8 qreg[NSTEP];
+    {
+      const T *qp = static_cast<const T *>(p.q) + seq * p.q_stride + (int64_t)qh * HD;
+#pragma unroll
+      for (int s = 0; s < NSTEP; s++) {
+        const int ch = 4 * s + kg;
+        u32x4_t raw = {0u, 0u, 0u, 0u};
+        if (col_ok && ch < NCH) raw = *reinterpret_cast<const u32x4_t *>(qp + ch * 8);
+        qreg[s] = bit_cast<vec8>(raw);
+      }
+    }
+    const float slope = (p.alibi != nullptr && col_ok) ? p.alibi[qh] * kLog2e : 0.f;
+    const T *kbase = static_cast<const T *>(p.kc) + (int64_t)kvh * p.k_head_stride;
+    const T *vbase = static_cast<const T *>(p.vc) + (int64_t)kvh * p.v_head_stride;
+
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4_t acc[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // The table entries of up to 32 pairs sit one per lane.
+    for (int sp = 0; sp < n; sp += 32) {
+      const int nsub = min(32, n - sp);
+      const int b_first = 2 * (pr0 + sp);
+      int tbl = 0;
+      if (b_first + lane < p.table_cols) tbl = p.block_tables[seq * p.max_blocks + b_first + lane];
+      // Two register sets (heads up to 128 elements): the next pair's loads are
+      // in flight while the current pair is folded in.
+      auto issue = [&](int it, PairRegs<HD> &r) {
+        const bool has_b = b_first + 2 * it + 1 < nblk;
+        const int64_t pa = __builtin_amdgcn_readlane(tbl, 2 * it);
+        const int64_t pb = __builtin_amdgcn_readlane(tbl, has_b ? 2 * it + 1 : 2 * it);
+        pair_load<T, HD>(p, kbase, vbase, pa, pb, r);
+      };
+      auto fold = [&](int it, PairRegs<HD> &r) {
+        const int blk = b_first + 2 * it;
+        pair_compute<T, HD>(p, r, blk, blk + 1 < nblk, ctx, slope, qreg, m_run, l_run, acc);
+      };
+      if (HD <= 128) {
+        PairRegs<HD> ra, rb;
+        issue(0, ra);
+        for (int it = 0; it < nsub; it += 2) {
+          if (it + 1 < nsub) issue(it + 1, rb);
+          fold(it, ra);
+          if (it + 1 < nsub) {
+            if (it + 2 < nsub) issue(it + 2, ra);
+            fold(it + 1, rb);
+          }
+        }
+      } else {  // two register sets of 256-element heads do not fit
+        for (int it = 0; it < nsub; it++) {
+          PairRegs<HD> ra;
+          issue(it, ra);
+          fold(it, ra);
+        }
+      }
+    }
+
+    float l_tot = l_run + __shfl_xor(l_run, 16, 64);
+    l_tot += __shfl_xor(l_tot, 32, 64);
+    if (col_ok) {
+      if (pr0 == 0 && n == pairs) {
+        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        T *op = out + seq * p.out_stride + (int64_t)qh * HD + kg * 4;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) {
+          T rr[4];
+#pragma unroll
+          for (int i = 0; i < 4; i++) rr[i] = from_float<T>(acc[dt][i] * inv);
+          *reinterpret_cast<u32x2_t *>(op + dt * 16) = *reinterpret_cast<u32x2_t *>(rr);
+        }
+      } else {
+        const int64_t pidx = (int64_t)(2 * w + (u != u_first ? 1 : 0)) * p.flat_cols + col;
+        float *ap = p.ws_acc + pidx * HD + kg * 4;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) *reinterpret_cast<f32x4_t *>(ap + dt * 16) = acc[dt];
+        if (kg == 0) {
+          p.ws_m[pidx] = m_run;
+          p.ws_l[pidx] = l_tot;
+        }
+      }
+    }
+    u += n;
+    if (pr0 + n == pairs && h == hk - 1) seq++;
+  }
+}
+
+// Merge for the flat split: grid (Hq, S).  The wavefronts that cover the
+// segment of (sequence, kv head) follow from the unit arithmetic of the main
+// kernel; a segment covered by one wavefront was already written.
+template <typename T, int HD>
+__global__ __launch_bounds__(128) void paged_decode_flat_reduce_kernel(DecodeParams p) {
+  const int qh = blockIdx.x, seq = blockIdx.y;
+  const int lane = threadIdx.x & 63;
+  const int before = p.flat_prefix[seq];
+  const int pairs = p.flat_prefix[seq + 1] - before;
+  T *op = static_cast<T *>(p.out) + seq * p.out_stride + (int64_t)qh * HD;
+  if (pairs == 0) {  // empty context: nobody else writes the row
+    for (int d = threadIdx.x; d < HD; d += blockDim.x) op[d] = from_float<T>(0.f);
+    return;
+  }
+  const int hk = p.Hkv * p.col_groups;
+  const int total_units = hk * p.flat_prefix[p.num_seqs];
+  const FlatSplit split(total_units, p.flat_waves);
+  const int kvh = qh / p.G;
+  const int g_idx = qh - kvh * p.G;
+  const int h = kvh * p.col_groups + g_idx / 16;
+  const int col = g_idx % 16;
+  const int u0 = hk * before + h * pairs;
+  const int w0 = split.wave_of(u0);
+  const int w1 = split.wave_of(u0 + pairs - 1);
+  if (w0 == w1) return;
+  const int np = w1 - w0 + 1;
+  const int first_odd = u0 > split.start(w0) ? 1 : 0;
+  // slot of piece i: wavefront w0 + i; only the first piece can start inside its wavefront's range
+  auto slot = [&](int i) -> int64_t { return (int64_t)(2 * (w0 + i) + (i == 0 ? first_odd : 0)) * p.flat_cols + col; };
+  float mmax = -INFINITY;
+  for (int i = lane; i < np; i += 64) mmax = fmaxf(mmax, p.ws_m[slot(i)]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mmax = fmaxf(mmax, __shfl_xor(mmax, o, 64));
+  float denom = 0.f;
+  for (int i = lane; i < np; i += 64) denom += p.ws_l[slot(i)] * fast_exp2(p.ws_m[slot(i)] - mmax);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) denom += __shfl_xor(denom, o, 64);
+  const float inv = denom > 0.f ? 1.0f / denom : 0.f;
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    float o = 0.f;
+#pragma unroll 4
+    for (int i = 0; i < np; i++) o += p.ws_acc[slot(i) * HD + d] * fast_exp2(p.ws_m[slot(i)] - mmax);
+    op[d] = from_float<T>(o * inv);
+  }
+}
+
+// Workgroups of the flat launch: what the device holds at once (times a small
+// oversubscription factor), but no more than gives every wavefront
+// `min_chunk` units of the largest possible step.
+template <typename T, int HD>
+int flat_workgroups(int64_t max_units) {
+  static int resident = 0;  // workgroups of this kernel the current device holds
+  if (resident == 0) {
+    int dev = 0, per_cu = 0;
+    hipDeviceProp_t prop;
+    HA_HIP(hipGetDevice(&dev));
+    HA_HIP(hipGetDeviceProperties(&prop, dev));
+    HA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, paged_decode_flat_kernel<T, HD>, 256, 0));
+    resident = (per_cu > 0 ? per_cu : 1) * prop.multiProcessorCount;
+  }
+  int64_t wgs = resident;
+  if (const char *e = getenv("HIPATTN_DECODE_FLAT_WGS")) {
+    const int v = atoi(e);
+    if (v > 0) wgs = v;
+  }
+  const int64_t min_chunk = 2;
+  const int64_t cap = (max_units + 4 * min_chunk - 1) / (4 * min_chunk);
+  if (wgs > cap) wgs = cap;
+  return (int)(wgs < 1 ? 1 : wgs);
+}
+
+template <typename T, int HD>
+void launch_decode_flat(DecodeParams p, int64_t S, int max_context_len, hipStream_t stream) {
+  const int64_t max_units = S * p.Hkv * p.col_groups * ((max_context_len + 2 * kBlockSize - 1) / (2 * kBlockSize));
+  const int wgs = flat_workgroups<T, HD>(max_units);
+  p.flat_waves = wgs * 4;
+  p.flat_cols = p.G < 16 ? p.G : 16;
+  const size_t slots = (size_t)2 * p.flat_waves * p.flat_cols;
+  const size_t prefix_bytes = (((size_t)S + 1) * sizeof(int) + 255) & ~(size_t)255;
+  char *ws = static_cast<char *>(library_workspace(prefix_bytes + slots * (HD + 2) * sizeof(float), stream));
+  p.flat_prefix = reinterpret_cast<int *>(ws);
+  p.ws_acc = reinterpret_cast<float *>(ws + prefix_bytes);
+  p.ws_m = p.ws_acc + slots * HD;
+  p.ws_l = p.ws_m + slots;
+  paged_decode_flat_kernel<T, HD><<<dim3((unsigned)wgs), 256, 0, stream>>>(p);
+  check_launch("paged_attention");
+  paged_decode_flat_reduce_kernel<T, HD><<<dim3((unsigned)p.Hq, (unsigned)S), HD <= 64 ? 64 : 128, 0, stream>>>(p);
+  check_launch("paged_attention reduce");
+}
+
+template <typename T>
+void dispatch_head_flat(const DecodeParams &p, int head_size, int64_t S, int max_context_len, hipStream_t stream) {
+  switch (head_size) {
+    case 64: launch_decode_flat<T, 64>(p, S, max_context_len, stream); break;
+    case 80: launch_decode_flat<T, 80>(p, S, max_context_len, stream); break;
+    case 96: launch_decode_flat<T, 96>(p, S, max_context_len, stream); break;
+    case 112: launch_decode_flat<T, 112>(p, S, max_context_len, stream); break;
+    case 128: launch_decode_flat<T, 128>(p, S, max_context_len, stream); break;
+    case 256: launch_decode_flat<T, 256>(p, S, max_context_len, stream); break;
+    default: fail("paged_attention: unsupported head size %d (supported: 64, 80, 96, 112, 128, 256)", head_size);
+  }
+}
+
+// v1 takes the flat split for long steps: measured on MI355X it wins a few
+// percent once every wavefront of the launch has tens of block pairs to
+// stream, and loses to the partitioned launch (whose many short workgroups
+// hide the per-segment load chains behind each other) on short contexts or
+// small batches.  Its bookkeeping also needs the sequence table to fit in LDS
+// and unit indices in 32 bits.  HIPATTN_DECODE_FLAT=0/1 forces the choice
+// (tuning aid).
+bool use_flat_split(int64_t S, int hk, int max_context_len) {
+  if (S > kFlatMaxSeqs || max_context_len <= 0) return false;
+  const int64_t max_units = S * hk * ((max_context_len + 2 * kBlockSize - 1) / (2 * kBlockSize));
+  if (max_units >= (int64_t)1 << 30) return false;
+  if (const char *e = getenv("HIPATTN_DECODE_FLAT")) return atoi(e) != 0;
+  return max_context_len >= 1024 && max_units >= 32 * 2048;
 }
 
 // Partition length used by v1, in KV blocks: a multiple of 8 (one block pair
@@ -520,6 +902,12 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
     p.ws_l = static_cast<float *>(exp_sums->data);
     p.ws_m = static_cast<float *>(max_logits->data);
     p.tmp_out = tmp_out->data;
+  } else if (use_flat_split(S, p.Hkv * p.col_groups, max_context_len)) {
+    if (query->dtype == HIPATTN_F16)
+      dispatch_head_flat<half_t>(p, hd, S, max_context_len, stream);
+    else
+      dispatch_head_flat<bf16_t>(p, hd, S, max_context_len, stream);
+    return;
   } else {
     p.part_blocks = choose_part_blocks(S, p.Hkv, p.col_groups, max_context_len);
     int64_t P = (max_blocks + p.part_blocks - 1) / p.part_blocks;
