@@ -68,6 +68,70 @@ def cpu_baseline_decode(c_cpu, rows, threads: int) -> dict:
                       "bytes counted as for the GPU (bf16 K/V once per kv head)"}
 
 
+def llama_step_leg(dev, stream, steps: int, layers: int, share_cache: bool) -> dict:
+    """One full engine step of a Llama-3-8B-shaped model (random weights): 128 sequences decoding
+    one token each over contexts U[1024,16384] (seed 5), every layer with its own paged KV cache,
+    then the AICI step (5 % of the vocabulary allowed per sequence, packed bit masks) and greedy
+    arg-max.  Projections are library GEMMs; everything else runs through the C ABI."""
+    import numpy as np
+    import torch
+
+    from aici_amd import llama, paged
+    from aici_amd import workloads as W
+
+    cfg = llama.LlamaConfig.llama3_8b()
+    cfg.num_hidden_layers = layers
+    rng = np.random.default_rng(5)
+    S = 128
+    ctx = rng.integers(1024, 16384 + 1, size=S)
+    pool = int(((ctx + 15) // 16).sum()) + 64
+    alloc = paged.BlockAllocator(16, pool)
+    builder = paged.BatchInfoBuilder(16, cfg.max_position_embeddings, 1)
+    for sid, n in enumerate(ctx.tolist(), start=1):
+        alloc.alloc_seq(sid, n)
+        builder.sched_out(alloc, sid, rng.integers(0, cfg.vocab_size, size=n).astype(np.int32), n - 1)
+    bi = builder.finish().to(dev)
+    model = llama.Llama(cfg, llama.random_weights(cfg, 5, device=dev), dev)
+    g = torch.Generator(device=dev).manual_seed(5)
+    caches = []
+    for i in range(layers):
+        if share_cache and i > 0:
+            caches.append(caches[0])
+            continue
+        kc, vc = paged.alloc_gpu_cache_layer(pool, cfg.num_key_value_heads, cfg.head_dim, 16, cfg.dtype, dev)
+        kc.normal_(generator=g)
+        vc.normal_(generator=g)
+        caches.append((kc, vc))
+    allowed = W.allow_mask(5, S, cfg.vocab_size)
+    masks = torch.from_numpy(np.packbits(np.pad(allowed, ((0, 0), (0, (-cfg.vocab_size) % 32))), axis=1,
+                                         bitorder="little")).to(dev)
+
+    def step():
+        return llama.aici_greedy(model.forward(bi, caches), masks)
+
+    for _ in range(2):
+        toks = step()
+    torch.cuda.synchronize()
+    ok = bool(torch.from_numpy(allowed)[torch.arange(S), toks.cpu().long()].all())
+    ms = event_times_ms(step, steps, stream)
+    ms = sum(ms) / len(ms)
+    elt = 2
+    kv_bytes = int(ctx.sum()) * 2 * cfg.num_key_value_heads * cfg.head_dim * elt * layers
+    H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    kvd = cfg.num_key_value_heads * cfg.head_dim
+    weight_bytes = elt * (layers * (H * (H + 2 * kvd) + H * H + 3 * H * I) + V * H)
+    return {"ms_per_step": round(ms, 3), "steps": steps, "tokens_per_s": round(S / (ms * 1e-3), 1),
+            "kv_bytes_per_step": kv_bytes, "weight_bytes_per_step": weight_bytes,
+            "hbm_gbs": round((kv_bytes + weight_bytes) / (ms * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round((kv_bytes + weight_bytes) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "constrained_tokens_all_allowed": ok,
+            "config": {"workload": f"Llama-3-8B-shaped decode step, {layers} layers, 128 seqs, ctx U[1024,16384] "
+                                   "(seed 5), bf16, per-layer paged KV"
+                                   + (" (one cache shared by all layers)" if share_cache else "")
+                                   + ", AICI 5% allow-mask + greedy",
+                       "context_tokens": int(ctx.sum())}}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -76,6 +140,11 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--kv-pools", type=int, default=3, help="copies of the KV pool cycled through by the decode leg")
+    ap.add_argument("--llama-step", action="store_true",
+                    help="also time a full Llama-3-8B-shaped decode step with the AICI mask + greedy stage "
+                         "(allocates about 170 GB of HBM)")
+    ap.add_argument("--llama-layers", type=int, default=32)
+    ap.add_argument("--llama-share-cache", action="store_true", help="all layers read one layer's KV cache")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (torch copy_) so that FETCH_SIZE / WRITE_SIZE "
                          "read under rocprofv3 --pmc can be scaled against a kernel of known traffic")
@@ -179,6 +248,13 @@ def main() -> None:
                          "kernel": "prefill_varlen_kernel, HIP events"},
         }
         del p
+
+    # ---- optional: the full engine step the decode kernel sits in ---------------------------------
+    if args.llama_step:
+        del pools, c
+        torch.cuda.empty_cache()
+        line["llama_step"] = llama_step_leg(dev, stream, max(3, min(args.steps, 10)), args.llama_layers,
+                                            args.llama_share_cache)
 
     # ---- CPU baseline: the reference's CPU route on this box's host cores ------------------------
     if not args.no_cpu_baseline:
