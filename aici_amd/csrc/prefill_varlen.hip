@@ -78,6 +78,14 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 // max(a, b, c) in one instruction.  Scores are never NaN here, so the
 // canonicalising copies fmaxf would add to every MFMA result are not needed.
+// Maximum of a value and its counterpart in the other half of the wavefront
+// (lane ^ 32), through the gfx950 half-swap instead of an LDS permute.
+__device__ __forceinline__ float max_across_halves(float x) {
+  const unsigned u = bit_cast<unsigned>(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(bit_cast<float>((unsigned)r[0]), bit_cast<float>((unsigned)r[1]));
+}
+
 __device__ __forceinline__ float max3(float a, float b, float c) {
   float r;
   asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
@@ -262,7 +270,7 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
           float mx = s[qt][0];
 #pragma unroll
           for (int i = 1; i < 16; i++) mx = fmaxf(mx, s[qt][i]);
-          mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * p.scale_log2;
+          mx = max_across_halves(mx) * p.scale_log2;
           const bool grow = mx > m_run[qt] + kRescaleThreshold;
           if (__builtin_expect(__any(grow), 0)) {
             const float m_new = grow ? mx : m_run[qt];
@@ -583,7 +591,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
     for (int i = 1; i < 16; i++) mx = max3(mx, s[0][i], s[1][i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * p.scale_log2;
+    mx = max_across_halves(mx) * p.scale_log2;
     const bool grow = mx > m_run + kRescaleThreshold;
     if (__builtin_expect(__any(grow), 0)) {
       const float m_new = grow ? mx : m_run;
