@@ -33,8 +33,27 @@
 // error (2^-9 relative in bf16, 2^-12 in fp16); the normaliser is given the
 // same rounding for each half-tile's largest term so that it cancels where it
 // matters, on rows that one key dominates.
+#include <type_traits>
+
 #include "common.h"
 #include "device_types.h"
+
+// Phase timeline of one workgroup of the eight-wavefront kernel: built with
+// -DHIPATTN_PHASE_TRACE=<workgroup id>, lane 0 of every wavefront of that
+// workgroup stores the constant-rate 100 MHz counter at the phase boundaries
+// of its first 64 tiles; hipattn_debug_phase_trace copies the table out.  Not
+// compiled into normal builds.
+#ifdef HIPATTN_PHASE_TRACE
+__device__ long long g_phase_trace[64 * 8 * 8];
+#define PHASE_STAMP(slot)                                                                                        \
+  do {                                                                                                           \
+    if (blockIdx.x == HIPATTN_PHASE_TRACE && j < 64 && lane == 0) g_phase_trace[(j * 8 + wave) * 8 + (slot)] = wall_clock64(); \
+  } while (0)
+#else
+#define PHASE_STAMP(slot) \
+  do {                    \
+  } while (0)
+#endif
 
 namespace hipattn {
 
@@ -78,6 +97,14 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 // max(a, b, c) in one instruction.  Scores are never NaN here, so the
 // canonicalising copies fmaxf would add to every MFMA result are not needed.
+// Workgroup barrier for LDS hand-offs: waits for this wavefront's LDS
+// operations only.  __syncthreads() also drains the vector-memory counter,
+// which would make every tile wait for the global loads of the tile after next
+// that were just issued.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // Maximum of a value and its counterpart in the other half of the wavefront
 // (lane ^ 32), through the gfx950 half-swap instead of an LDS permute.
 __device__ __forceinline__ float max_across_halves(float x) {
@@ -470,25 +497,26 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   u32x2_t vst[NLOADV][4];
   const int v_dg = (wave & 3) * 8 + (lane & 7);        // 4-element group of the head dimension
   const int v_kg4 = (wave >> 2) * 8 + (lane >> 3);     // 4-key group of the tile, 0..15
-  // Per-thread element offsets inside a tile, relative to its first key; a
-  // full tile only adds the tile's base (one 64-bit add per load).
-  int64_t k_toff[NLOADK], v_toff[4];
+  // Per-thread byte offsets inside a tile, relative to its first key, in 32
+  // bits (the launcher checks that 64 rows fit): a full tile's loads are then
+  // a uniform base plus a 32-bit lane offset.
+  uint32_t k_boff[NLOADK];
 #pragma unroll
   for (int i = 0; i < NLOADK; i++) {
     const int idx = min(tid + 512 * i, K_CHUNKS - 1);
-    k_toff[i] = (int64_t)(idx / CPR) * p.k_row + min(idx % CPR, d_chunks - 1) * 8;
+    k_boff[i] = (uint32_t)(((int64_t)(idx / CPR) * p.k_row + min(idx % CPR, d_chunks - 1) * 8) * (int64_t)sizeof(T));
   }
-#pragma unroll
-  for (int kk = 0; kk < 4; kk++) v_toff[kk] = (int64_t)(v_kg4 * 4 + kk) * p.v_row + min(v_dg, p.d / 4 - 1) * 4;
+  const uint32_t v_boff = (uint32_t)(((int64_t)(v_kg4 * 4) * p.v_row + min(v_dg, p.d / 4 - 1) * 4) * (int64_t)sizeof(T));
   auto load_tile = [&](int tile) {
     const int k0 = tile * BN;
     if (k0 + BN <= Lk) {
-      const T *kt = kp + (int64_t)k0 * p.k_row;
-      const T *vt = vp + (int64_t)k0 * p.v_row;
+      const char *kt = reinterpret_cast<const char *>(kp + (int64_t)k0 * p.k_row);
+      const char *vt = reinterpret_cast<const char *>(vp + (int64_t)k0 * p.v_row);
 #pragma unroll
-      for (int i = 0; i < NLOADK; i++) kst[i] = *reinterpret_cast<const u32x4_t *>(kt + k_toff[i]);
+      for (int i = 0; i < NLOADK; i++) kst[i] = *reinterpret_cast<const u32x4_t *>(kt + k_boff[i]);
 #pragma unroll
-      for (int kk = 0; kk < 4; kk++) vst[0][kk] = *reinterpret_cast<const u32x2_t *>(vt + v_toff[kk]);
+      for (int kk = 0; kk < 4; kk++)
+        vst[0][kk] = *reinterpret_cast<const u32x2_t *>(vt + (int64_t)kk * p.v_row * (int64_t)sizeof(T) + v_boff);
     } else {  // the last, partial tile: clamp every key to the last real one
 #pragma unroll
       for (int i = 0; i < NLOADK; i++) {
@@ -546,9 +574,8 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   const int v_lane_off = c * TL::VTSTR + g * 8;
   const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  // ---- the three phases of one 64-key tile ------------------------------------
-  // Q: S^T = K . Q^T for both 32-key halves; LDS reads run two contraction
-  // steps ahead of the MFMAs that consume them.
+  // S^T = K . Q^T of one tile on its own (used for tile 0): both 32-key halves,
+  // LDS reads two contraction steps ahead of the MFMAs that consume them.
   auto phase_qk = [&](int buf, f32x16_t(&s)[2]) {
     const T *ks_base = smem + buf * TL::STAGE_ELEMS;
     auto rd = [&](int kt, int ks) -> vec8 {
@@ -573,8 +600,43 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  // S: mask, running maximum (moved lazily), exponentials -> MFMA operands.
-  auto phase_softmax = [&](int k0, f32x16_t(&s)[2], vec8(&pk)[2][2]) {
+  // Tiles entirely past the diagonal of every row of this wavefront are skipped.
+  auto skip_tile = [&](int j) { return (wave_row0 >= Lq) || (p.causal && j * BN > wave_last_row + off); };
+
+  // ---- the pipelined tile loop -------------------------------------------------
+  // Iteration j of a wavefront: the matrix pipe computes S(j+1) = K(j+1).Q^T while
+  // the vector ALU turns S(j) into probabilities -- one MFMA is issued, then the
+  // few softmax instructions that fit in its shadow, and so on -- then P(j).V(j)
+  // runs with the staging of tile j+2 (registers -> LDS) and the loads of tile
+  // j+3 in its shadow.  Three LDS buffers: iteration j reads K of (j+1)%3 and V
+  // of j%3 and writes (j+2)%3; one barrier per iteration.
+  constexpr int NQ = 2 * KSTEPS;   // MFMAs of one S tile: step n = (contraction step n/2, key half n%2)
+  constexpr int MAXS = NQ / 4;     // of which the first MAXS shadow the row maximum,
+  constexpr int EXPS = NQ - MAXS;  // the rest the exponentials
+  constexpr int QK_DEPTH = 3;      // K operands read ahead of their MFMA
+
+  // DO_QK: S(j+1) is wanted (written to sn); the softmax of S(j) (in s) always runs.
+  auto qk_softmax = [&](auto do_qk, int j, f32x16_t(&s)[2], f32x16_t(&sn)[2], vec8(&pk)[2][2]) {
+    constexpr bool DO_QK = decltype(do_qk)::value;
+    const int k0 = j * BN;
+    const T *ks_base = smem + ((j + 1) % 3) * TL::STAGE_ELEMS;
+    auto rd = [&](int n) -> vec8 {
+      return *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + (n & 1) * 32 * TL::KSTR + (n >> 1) * 16);
+    };
+    vec8 ka[QK_DEPTH + 1];
+    if (DO_QK) {
+#pragma unroll
+      for (int n = 0; n < QK_DEPTH && n < NQ; n++) ka[n] = rd(n);
+    }
+    auto qk_step = [&](int n) {
+      if (DO_QK) {
+        if (n + QK_DEPTH < NQ) ka[(n + QK_DEPTH) % (QK_DEPTH + 1)] = rd(n + QK_DEPTH);
+        __builtin_amdgcn_sched_barrier(0);
+        sn[n & 1] = Mfma32<T>::run(ka[n % (QK_DEPTH + 1)], qreg[n >> 1], (n >> 1) == 0 ? zero : sn[n & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+
     const bool need_mask = (k0 + BN > Lk) || (p.causal && k0 + BN - 1 > wave_row0 + off);
     if (need_mask) {
       const int row = wave_row0 + c;
@@ -588,9 +650,15 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
           if (key > limit) s[kt][i] = -INFINITY;
         }
     }
+    // row maximum in the shadow of the first MAXS MFMAs
     float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
-    for (int i = 1; i < 16; i++) mx = max3(mx, s[0][i], s[1][i]);
+    for (int n = 0; n < MAXS; n++) {
+      qk_step(n);
+#pragma unroll
+      for (int i = 16 * n / MAXS; i < 16 * (n + 1) / MAXS; i++)
+        if (i > 0) mx = max3(mx, s[0][i], s[1][i]);
+    }
     mx = max_across_halves(mx) * p.scale_log2;
     const bool grow = mx > m_run + kRescaleThreshold;
     if (__builtin_expect(__any(grow), 0)) {
@@ -604,78 +672,77 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     const float msub = m_run == -INFINITY ? 0.f : m_run;
     const float pmax = fast_exp2(mx - msub);
     float psum = g == 0 ? to_float(from_float<T>(pmax)) - pmax : 0.f;
+    // exponentials in the shadow of the remaining MFMAs; value v = (key half, register)
 #pragma unroll
-    for (int kt = 0; kt < 2; kt++)
+    for (int n = 0; n < EXPS; n++) {
+      qk_step(MAXS + n);
 #pragma unroll
-      for (int half = 0; half < 2; half++) {
-        vec8 v;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-          const float e = fast_exp2(s[kt][half * 8 + i] * p.scale_log2 - msub);
-          psum += e;
-          v[i] = from_float<T>(e);
-        }
-        pk[kt][half] = v;
+      for (int v = 32 * n / EXPS; v < 32 * (n + 1) / EXPS; v++) {
+        const float e = fast_exp2(s[v / 16][v % 16] * p.scale_log2 - msub);
+        psum += e;
+        pk[v / 16][(v % 16) / 8][v % 8] = from_float<T>(e);
       }
+    }
     l_run += psum;
   };
-  // P: O^T += V^T . P^T; step n = (dt, kt, half), its operand is read four steps ahead.
-  auto phase_pv = [&](int buf, vec8(&pk)[2][2]) {
-    const T *vs_base = smem + buf * TL::STAGE_ELEMS + TL::K_ELEMS;
-    constexpr int NSTEP = NDT * 4;
+
+  // P(j).V(j) with the staging for later tiles in its shadow.
+  constexpr int PV_STEPS = NDT * 4;  // step n = (dt, kt, half)
+  auto pv_stage = [&](bool live, int j, vec8(&pk)[2][2]) {
+    const T *vs_base = smem + (j % 3) * TL::STAGE_ELEMS + TL::K_ELEMS;
     auto rd = [&](int n) -> vec8 {
       const int dt = n / 4, kt = (n / 2) % 2, half = n % 2;
       return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + dt * 32 * TL::VTSTR + kt * 32 + half * 16);
     };
-    vec8 va[5];
+    if (live) {
+      vec8 va[4];
 #pragma unroll
-    for (int n = 0; n < 4 && n < NSTEP; n++) va[n] = rd(n);
+      for (int n = 0; n < 3 && n < PV_STEPS; n++) va[n] = rd(n);
 #pragma unroll
-    for (int n = 0; n < NSTEP; n++) {
-      if (n + 4 < NSTEP) va[(n + 4) % 5] = rd(n + 4);
-      __builtin_amdgcn_sched_barrier(0);
-      acc[n / 4] = Mfma32<T>::run(va[n % 5], pk[(n / 2) % 2][n % 2], acc[n / 4]);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int n = 0; n < PV_STEPS; n++) {
+        if (n + 3 < PV_STEPS) va[(n + 3) % 4] = rd(n + 3);
+        __builtin_amdgcn_sched_barrier(0);
+        acc[n / 4] = Mfma32<T>::run(va[n % 4], pk[(n / 2) % 2][n % 2], acc[n / 4]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (n == 1) {
+          if (j + 2 < n_tiles) store_tile((j + 2) % 3);
+          if (j + 3 < n_tiles) load_tile(j + 3);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    } else {
+      if (j + 2 < n_tiles) store_tile((j + 2) % 3);
+      if (j + 3 < n_tiles) load_tile(j + 3);
     }
   };
-  // Tiles entirely past the diagonal of every row of this wavefront are skipped.
-  auto skip_tile = [&](int j) { return (wave_row0 >= Lq) || (p.causal && j * BN > wave_last_row + off); };
 
-  // The two wavefronts that share a SIMD run the phases in different orders
-  // between two workgroup barriers -- wavefronts 0-3: Q S P of tile j;
-  // wavefronts 4-7: P of tile j-1, then Q S of tile j -- so that one is on the
-  // vector ALU while the other is on the matrix pipe instead of both queueing
-  // for the same unit.  V of tile j-1 must therefore survive iteration j:
-  // three tile buffers.
-  if (wave < 4) {
-    for (int j = 0; j < n_tiles; j++) {
-      if (j + 1 < n_tiles) store_tile((j + 1) % 3);
-      if (j + 2 < n_tiles) load_tile(j + 2);
-      if (!skip_tile(j)) {
-        f32x16_t s[2];
-        vec8 pk[2][2];
-        phase_qk(j % 3, s);
-        phase_softmax(j * BN, s, pk);
-        phase_pv(j % 3, pk);
-      }
-      __syncthreads();
-    }
-  } else {
+  f32x16_t s_a[2], s_b[2];
+  // S(0) has nothing to hide behind; tile 1 is staged while it runs.
+  if (n_tiles > 0 && !skip_tile(0)) phase_qk(0, s_a);
+  if (n_tiles > 1) store_tile(1);
+  if (n_tiles > 2) load_tile(2);
+  lds_barrier();
+
+  auto iteration = [&](int j, f32x16_t(&s)[2], f32x16_t(&sn)[2]) {
+    const bool live = !skip_tile(j);
+    const bool live_next = j + 1 < n_tiles && !skip_tile(j + 1);
     vec8 pk[2][2];
-    bool pending = false;
-    for (int j = 0; j < n_tiles; j++) {
-      if (j + 1 < n_tiles) store_tile((j + 1) % 3);
-      if (j + 2 < n_tiles) load_tile(j + 2);
-      if (pending) phase_pv((j + 2) % 3, pk);  // tile j-1
-      pending = !skip_tile(j);
-      if (pending) {
-        f32x16_t s[2];
-        phase_qk(j % 3, s);
-        phase_softmax(j * BN, s, pk);
-      }
-      __syncthreads();
+    PHASE_STAMP(0);
+    if (live) {
+      if (live_next)
+        qk_softmax(std::true_type{}, j, s, sn, pk);
+      else
+        qk_softmax(std::false_type{}, j, s, sn, pk);
     }
-    if (pending) phase_pv((n_tiles + 2) % 3, pk);  // tile n_tiles-1
+    PHASE_STAMP(1);
+    pv_stage(live, j, pk);
+    PHASE_STAMP(2);
+    lds_barrier();
+    PHASE_STAMP(3);
+  };
+  for (int j = 0; j < n_tiles; j += 2) {
+    iteration(j, s_a, s_b);
+    if (j + 1 < n_tiles) iteration(j + 1, s_b, s_a);
   }
 
   // ---- epilogue ---------------------------------------------------------------
@@ -742,8 +809,9 @@ void pick_qt(const PrefillParams &p, int64_t total_q, hipStream_t stream) {
   if constexpr (HDP <= 128) {
     const int64_t wg256 = (total_q / 256 + p.batch) * p.Hq;
     const char *force = getenv("HIPATTN_PREFILL_KERNEL");  // tuning aid: "w8", "qt2" or "qt1"
-    const bool big = wg256 >= 2 * 256;
-    if (force ? !strcmp(force, "w8") : big) {
+    // the eight-wavefront kernel addresses a tile's 64 rows with 32-bit byte offsets
+    const bool big = wg256 >= 2 * 256 && p.k_row < (1 << 23) && p.v_row < (1 << 23);
+    if ((force ? !strcmp(force, "w8") : big) && p.k_row < (1 << 23) && p.v_row < (1 << 23)) {
       launch_prefill_w8<T, HDP>(p, stream);
       return;
     }
@@ -899,3 +967,9 @@ extern "C" char *hipattn_mha_varlen_fwd(const hipattn_tensor *q, const hipattn_t
                                  softmax_scale, zero_tensors, is_causal, window_size_left, window_size_right, out,
                                  softmax_lse, stream));
 }
+
+#ifdef HIPATTN_PHASE_TRACE
+extern "C" int hipattn_debug_phase_trace(long long *dst, int n) {
+  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_phase_trace), sizeof(long long) * n);
+}
+#endif
