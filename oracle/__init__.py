@@ -23,7 +23,11 @@ How each function is pinned (tests/test_oracle_*.py):
   rms_norm               closed form in fp64 incl. the round-then-scale order;
   hostkv (allocator,     hand-computed cases from blocks.rs / batch_info.rs
   batch builder)         semantics plus exact agreement with the C++ core;
-  aici bias              bit order from aicirt/src/api.rs:278-292 on hand cases.
+  aici bias              bit order from aicirt/src/api.rs:278-292 on hand cases;
+  llama step             a composition of the functions above in the order of
+                         llama.rs; closed forms (zeroed output projections,
+                         one-token sequences) and prefill-then-decode ==
+                         one longer prefill (tests/test_oracle_llama.py).
 No function is left "parity unpinned" except the last-ulp behaviour of
 libtorch-CPU SDPA, which is irrelevant at the 5e-3 / 2e-2 gates and is
 bracketed by the fp64 brute force.
