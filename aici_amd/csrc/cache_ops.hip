@@ -65,6 +65,127 @@ __global__ __launch_bounds__(256) void cache_move_vec_kernel(
   }
 }
 
+// Runs of tokens (2-byte elements).  A workgroup takes 16 consecutive tokens in
+// two groups of 8.  When a group's slots are 8 consecutive offsets of one block starting at a
+// multiple of 8 -- the normal case of a prompt, whose tokens fill blocks in
+// order -- a thread moves an 8 token x 8 element tile of K and of V with
+// 16-byte accesses on both sides: K's eight runs are adjacent in the cache
+// (128 bytes), and V's tile is transposed in registers so that every head
+// element's eight tokens go out as one 16-byte run instead of eight 2-byte
+// stores 32 bytes apart.  Any other group (padding slots, block boundaries not
+// at multiples of 8, decode tokens) takes the per-token path of the kernel
+// above, its 8 tokens spread over the threads.
+template <typename Slot, bool SCATTER>
+__global__ __launch_bounds__(256) void cache_move_run8_kernel(
+    uint16_t *__restrict__ key, uint16_t *__restrict__ value, uint16_t *__restrict__ key_cache,
+    uint16_t *__restrict__ value_cache, const Slot *__restrict__ slot_mapping, int64_t num_tokens,
+    int64_t key_tok_stride, int64_t key_head_stride, int64_t val_tok_stride,
+    int64_t val_head_stride, CacheGeom g) {
+  typedef uint16_t E;
+  constexpr int X = 8;
+  // 16 tokens per workgroup, as two groups of 8: a block filled in order is then
+  // written by one workgroup, whose half-row stores meet in the same L2.
+  const int64_t wg_t0 = (int64_t)blockIdx.x * 16;
+  const int chunks_per_head = g.head_size / X;
+  const int n = g.num_heads * chunks_per_head;
+  int64_t run_slot[2];
+#pragma unroll
+  for (int half = 0; half < 2; half++) {
+    const int64_t t0 = wg_t0 + 8 * half;
+    run_slot[half] = -1;
+    if (t0 + 8 <= num_tokens) {
+      const int64_t slot0 = (int64_t)slot_mapping[t0];
+      bool run = slot0 >= 0 && slot0 % 8 == 0 && slot0 / g.block_size < g.num_blocks;
+      if (run) {
+#pragma unroll
+        for (int i = 1; i < 8; i++) run = run && (int64_t)slot_mapping[t0 + i] == slot0 + i;
+      }
+      if (run) run_slot[half] = slot0;
+    }
+  }
+  for (int idx = threadIdx.x; idx < 2 * n; idx += blockDim.x) {
+    const int half = idx / n;
+    const int i = idx % n;
+    const int h = i / chunks_per_head;
+    const int c = i % chunks_per_head;
+    const int64_t t0 = wg_t0 + 8 * half;
+    const int64_t slot0 = half == 0 ? run_slot[0] : run_slot[1];
+    if (slot0 >= 0) {
+      const int64_t blk = slot0 / g.block_size;
+      const int off0 = (int)(slot0 % g.block_size);
+      E *kp = key + t0 * key_tok_stride + h * key_head_stride + c * X;
+      E *vp = value + t0 * val_tok_stride + h * val_head_stride + c * X;
+      E *kc = key_cache + blk * g.k_block_stride + h * g.k_head_stride + ((int64_t)c * g.block_size + off0) * X;
+      E *vc = value_cache + blk * g.v_block_stride + h * g.v_head_stride + (int64_t)c * X * g.block_size + off0;
+      uint4 rows[8];
+      if (SCATTER) {
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+          *reinterpret_cast<uint4 *>(kc + t * X) = *reinterpret_cast<const uint4 *>(kp + t * key_tok_stride);
+#pragma unroll
+        for (int t = 0; t < 8; t++) rows[t] = *reinterpret_cast<const uint4 *>(vp + t * val_tok_stride);
+        const unsigned *r = reinterpret_cast<const unsigned *>(rows);  // r[4 t + k]: elements 2k, 2k+1 of token t
+#pragma unroll
+        for (int j = 0; j < 8; j++) {  // head element j of the chunk: tokens 0..7
+          const unsigned sel = (j & 1) ? 0x07060302u : 0x05040100u;
+          uint4 o;
+          o.x = __builtin_amdgcn_perm(r[4 * 1 + j / 2], r[4 * 0 + j / 2], sel);
+          o.y = __builtin_amdgcn_perm(r[4 * 3 + j / 2], r[4 * 2 + j / 2], sel);
+          o.z = __builtin_amdgcn_perm(r[4 * 5 + j / 2], r[4 * 4 + j / 2], sel);
+          o.w = __builtin_amdgcn_perm(r[4 * 7 + j / 2], r[4 * 6 + j / 2], sel);
+          *reinterpret_cast<uint4 *>(vc + (int64_t)j * g.block_size) = o;
+        }
+      } else {
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+          *reinterpret_cast<uint4 *>(kp + t * key_tok_stride) = *reinterpret_cast<const uint4 *>(kc + t * X);
+#pragma unroll
+        for (int j = 0; j < 8; j++) rows[j] = *reinterpret_cast<const uint4 *>(vc + (int64_t)j * g.block_size);
+        const unsigned *r = reinterpret_cast<const unsigned *>(rows);  // r[4 j + a]: tokens 2a, 2a+1 of element j
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          const unsigned sel = (t & 1) ? 0x07060302u : 0x05040100u;
+          uint4 o;
+          o.x = __builtin_amdgcn_perm(r[4 * 1 + t / 2], r[4 * 0 + t / 2], sel);
+          o.y = __builtin_amdgcn_perm(r[4 * 3 + t / 2], r[4 * 2 + t / 2], sel);
+          o.z = __builtin_amdgcn_perm(r[4 * 5 + t / 2], r[4 * 4 + t / 2], sel);
+          o.w = __builtin_amdgcn_perm(r[4 * 7 + t / 2], r[4 * 6 + t / 2], sel);
+          *reinterpret_cast<uint4 *>(vp + t * val_tok_stride) = o;
+        }
+      }
+      continue;
+    }
+    // per-token path for this group of 8
+    for (int t = 0; t < 8; t++) {
+      const int64_t token = t0 + t;
+      if (token >= num_tokens) break;
+      const int64_t slot = (int64_t)slot_mapping[token];
+      if (slot < 0) continue;
+      const int64_t blk = slot / g.block_size;
+      if (blk >= g.num_blocks) continue;
+      const int off = (int)(slot % g.block_size);
+      E *kp = key + token * key_tok_stride + h * key_head_stride + c * X;
+      E *vp = value + token * val_tok_stride + h * val_head_stride + c * X;
+      E *kc = key_cache + blk * g.k_block_stride + h * g.k_head_stride + ((int64_t)c * g.block_size + off) * X;
+      E *vc = value_cache + blk * g.v_block_stride + h * g.v_head_stride + (int64_t)c * X * g.block_size + off;
+      if (SCATTER) {
+        *reinterpret_cast<uint4 *>(kc) = *reinterpret_cast<const uint4 *>(kp);
+        uint4 vv = *reinterpret_cast<const uint4 *>(vp);
+        const E *ve = reinterpret_cast<const E *>(&vv);
+#pragma unroll
+        for (int j = 0; j < X; j++) vc[(int64_t)j * g.block_size] = ve[j];
+      } else {
+        *reinterpret_cast<uint4 *>(kp) = *reinterpret_cast<const uint4 *>(kc);
+        uint4 vv;
+        E *ve = reinterpret_cast<E *>(&vv);
+#pragma unroll
+        for (int j = 0; j < X; j++) ve[j] = vc[(int64_t)j * g.block_size];
+        *reinterpret_cast<uint4 *>(vp) = vv;
+      }
+    }
+  }
+}
+
 // Element-wise variant for rows that are not 16-byte aligned.
 template <typename E, typename Slot, bool SCATTER>
 __global__ __launch_bounds__(256) void cache_move_scalar_kernel(
@@ -147,6 +268,18 @@ void launch_move(const hipattn_tensor *key, const hipattn_tensor *value,
                    value->strides[1] % X == 0 && g.k_block_stride % X == 0 &&
                    g.k_head_stride % X == 0 && g.head_size % X == 0;
   dim3 grid((unsigned)T);
+  if constexpr (sizeof(E) == 2) {
+    // long inputs (prompts): 8-token workgroups with the transposing fast path
+    if (vec && T >= 1024 && g.block_size % 8 == 0 && aligned16(vc) && g.v_block_stride % 8 == 0 &&
+        g.v_head_stride % 8 == 0) {
+      int n = g.num_heads * (g.head_size / X);
+      int threads = n < 256 ? ((n + 63) / 64) * 64 : 256;
+      cache_move_run8_kernel<Slot, SCATTER><<<dim3((unsigned)((T + 15) / 16)), threads, 0, stream>>>(
+          kp, vp, kc, vc, sp, T, key->strides[0], key->strides[1], value->strides[0], value->strides[1], g);
+      check_launch(SCATTER ? "reshape_and_cache" : "gather_cached_kv");
+      return;
+    }
+  }
   if (vec) {
     int n = g.num_heads * (g.head_size / X);
     int threads = n < 256 ? ((n + 63) / 64) * 64 : 256;

@@ -3,6 +3,7 @@
 // accesses where alignment allows, reductions through wave shuffles and LDS.
 #include "common.h"
 #include "device_types.h"
+#include "workspace.h"
 
 namespace hipattn {
 
@@ -85,6 +86,44 @@ __global__ __launch_bounds__(512) void rotary_kernel(const Pos *__restrict__ pos
   }
 }
 
+// NeoX layout, 2-byte types, in 16-byte steps: a thread rotates 8 pairs
+// (x at r..r+7, y at rot/2 + r..) of one head.  Same per-operation rounding.
+template <typename T, typename Pos>
+__global__ __launch_bounds__(512) void rotary_neox_vec8_kernel(const Pos *__restrict__ positions, T *__restrict__ query,
+                                                               T *__restrict__ key, const T *__restrict__ cos_sin,
+                                                               int rot_dim, int64_t q_stride, int64_t k_stride,
+                                                               int num_heads, int num_kv_heads, int head_size,
+                                                               int64_t max_pos) {
+  const int64_t token = blockIdx.x;
+  const int64_t pos = (int64_t)positions[token];
+  if (pos < 0 || pos >= max_pos) return;
+  const int embed = rot_dim / 2;
+  const int per_head = embed / 8;
+  const int n = (num_heads + num_kv_heads) * per_head;
+  const T *cos_ptr = cos_sin + pos * rot_dim;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int hd = i / per_head;
+    const int r = (i % per_head) * 8;
+    T *arr = hd < num_heads ? query + token * q_stride + (int64_t)hd * head_size
+                            : key + token * k_stride + (int64_t)(hd - num_heads) * head_size;
+    const uint4 xr = *reinterpret_cast<const uint4 *>(arr + r);
+    const uint4 yr = *reinterpret_cast<const uint4 *>(arr + embed + r);
+    const uint4 cr = *reinterpret_cast<const uint4 *>(cos_ptr + r);
+    const uint4 sr = *reinterpret_cast<const uint4 *>(cos_ptr + embed + r);
+    const T *x = reinterpret_cast<const T *>(&xr), *y = reinterpret_cast<const T *>(&yr);
+    const T *c = reinterpret_cast<const T *>(&cr), *sn = reinterpret_cast<const T *>(&sr);
+    uint4 xo, yo;
+    T *xe = reinterpret_cast<T *>(&xo), *ye = reinterpret_cast<T *>(&yo);
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      xe[j] = sub_t(mul_t(x[j], c[j]), mul_t(y[j], sn[j]));
+      ye[j] = add_t(mul_t(y[j], c[j]), mul_t(x[j], sn[j]));
+    }
+    *reinterpret_cast<uint4 *>(arr + r) = xo;
+    *reinterpret_cast<uint4 *>(arr + embed + r) = yo;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // rms_norm / fused_add_rms_norm (layernorm_kernels.cu:10-65):
 //   out = T(x * rsqrt(mean(x^2) + eps)) * w, the product again rounded to T.
@@ -120,6 +159,63 @@ __global__ __launch_bounds__(1024) void rms_norm_kernel(T *__restrict__ out, T *
   }
 }
 
+// 16-byte variant for 2-byte types: a thread keeps its 8 elements in registers
+// between the reduction and the scaling, so every byte crosses once.
+template <typename T, bool FUSED_ADD>
+__global__ __launch_bounds__(1024) void rms_norm_vec8_kernel(T *__restrict__ out, T *__restrict__ input,
+                                                             T *__restrict__ residual,
+                                                             const T *__restrict__ weight, float eps, int hidden) {
+  __shared__ float smem[17];
+  const int64_t row = blockIdx.x;
+  const int i = threadIdx.x * 8;
+  const bool active = i < hidden;
+  T *x = input + row * (int64_t)hidden + i;
+  float v[8];
+  float ss = 0.f;
+  if (active) {
+    const uint4 raw = *reinterpret_cast<const uint4 *>(x);
+    const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = to_float(e[j]);
+    if (FUSED_ADD) {
+      T *res = residual + row * (int64_t)hidden + i;
+      const uint4 rr = *reinterpret_cast<const uint4 *>(res);
+      const T *re = reinterpret_cast<const T *>(&rr);
+      uint4 ro;
+      T *oe = reinterpret_cast<T *>(&ro);
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        v[j] += to_float(re[j]);
+        oe[j] = from_float<T>(v[j]);
+      }
+      *reinterpret_cast<uint4 *>(res) = ro;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        ss += v[j] * v[j];            // variance from the un-rounded sum,
+        v[j] = to_float(oe[j]);       // scaling from the rounded one (layernorm_kernels.cu:48-63)
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; j++) ss += v[j] * v[j];
+    }
+  }
+  const float total = block_sum(ss, smem);
+  const float inv = rsqrtf(total / (float)hidden + eps);
+  if (active) {
+    const uint4 wr = *reinterpret_cast<const uint4 *>(weight + i);
+    const T *we = reinterpret_cast<const T *>(&wr);
+    uint4 o;
+    T *oe = reinterpret_cast<T *>(&o);
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const T normed = from_float<T>(v[j] * inv);
+      oe[j] = from_float<T>(to_float(normed) * to_float(we[j]));
+    }
+    T *op = FUSED_ADD ? x : out + row * (int64_t)hidden + i;
+    *reinterpret_cast<uint4 *>(op) = o;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Activations (activation_kernels.cu:15-115).
 // ---------------------------------------------------------------------------
@@ -137,6 +233,22 @@ __global__ __launch_bounds__(1024) void silu_and_mul_kernel(T *__restrict__ out,
     const T y = in[row * 2 * d + d + i];
     out[row * d + i] = mul_t(silu_t(x), y);
   }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void silu_and_mul_vec8_kernel(T *__restrict__ out, const T *__restrict__ in, int d) {
+  const int64_t row = blockIdx.y;
+  const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (i >= d) return;
+  const uint4 xr = *reinterpret_cast<const uint4 *>(in + row * 2 * d + i);
+  const uint4 yr = *reinterpret_cast<const uint4 *>(in + row * 2 * d + d + i);
+  const T *xe = reinterpret_cast<const T *>(&xr);
+  const T *ye = reinterpret_cast<const T *>(&yr);
+  uint4 o;
+  T *oe = reinterpret_cast<T *>(&o);
+#pragma unroll
+  for (int j = 0; j < 8; j++) oe[j] = mul_t(silu_t(xe[j]), ye[j]);
+  *reinterpret_cast<uint4 *>(out + row * d + i) = o;
 }
 
 template <typename T>
@@ -230,6 +342,110 @@ __global__ __launch_bounds__(1024) void bias_argmax_kernel(const T *__restrict__
   }
 }
 
+// Wide variant: each row is cut into `chunks` slices handled by separate
+// workgroups (a step has far fewer sequences than the chip has CUs), 8 logits
+// and one mask byte per thread and load; a second small kernel picks the best
+// slice.  Same order rule: the largest value, the lowest id among equals.
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void bias_argmax_slice_kernel(const T *__restrict__ logits, int64_t logit_stride,
+                                                                const float *__restrict__ bias, int64_t bias_stride,
+                                                                const uint8_t *__restrict__ mask, int64_t mask_stride,
+                                                                int64_t mask_bytes, const int32_t *__restrict__ rows,
+                                                                int vocab, int per_slice /* multiple of 8 */,
+                                                                float *__restrict__ part_val,
+                                                                int32_t *__restrict__ part_idx) {
+  __shared__ float s_val[4];
+  __shared__ int s_idx[4];
+  const int64_t seq = blockIdx.y;
+  const int slice = blockIdx.x;
+  const int64_t row = rows ? (int64_t)rows[seq] : seq;
+  const T *lg = logits + seq * logit_stride;
+  const int begin = slice * per_slice;
+  const int end = min(begin + per_slice, vocab);
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int i = begin + threadIdx.x * 8; i < end; i += blockDim.x * 8) {
+    const uint4 raw = *reinterpret_cast<const uint4 *>(lg + i);
+    const T *e = reinterpret_cast<const T *>(&raw);
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = to_float(e[j]);
+    if (MODE == 0) {
+      const float4 b0 = *reinterpret_cast<const float4 *>(bias + row * bias_stride + i);
+      const float4 b1 = *reinterpret_cast<const float4 *>(bias + row * bias_stride + i + 4);
+      v[0] += b0.x; v[1] += b0.y; v[2] += b0.z; v[3] += b0.w;
+      v[4] += b1.x; v[5] += b1.y; v[6] += b1.z; v[7] += b1.w;
+    } else {
+      const int64_t byte = i >> 3;
+      const unsigned m = byte < mask_bytes ? mask[row * mask_stride + byte] : 0u;
+#pragma unroll
+      for (int j = 0; j < 8; j++)
+        if (!((m >> j) & 1)) v[j] = -INFINITY;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+      if (v[j] > best) {  // increasing ids within a thread: ties keep the lowest
+        best = v[j];
+        best_i = i + j;
+      }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(best_i, o, 64);
+    if (ov > best || (ov == best && oi < best_i)) {
+      best = ov;
+      best_i = oi;
+    }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    s_val[wave] = best;
+    s_idx[wave] = best_i;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < (int)(blockDim.x >> 6); w++)
+      if (s_val[w] > best || (s_val[w] == best && s_idx[w] < best_i)) {
+        best = s_val[w];
+        best_i = s_idx[w];
+      }
+    part_val[seq * gridDim.x + slice] = best;
+    part_idx[seq * gridDim.x + slice] = best_i;
+  }
+}
+
+__global__ __launch_bounds__(64) void bias_argmax_pick_kernel(const float *__restrict__ part_val,
+                                                              const int32_t *__restrict__ part_idx, int chunks,
+                                                              int32_t *__restrict__ out_tokens,
+                                                              float *__restrict__ out_logits) {
+  const int64_t seq = blockIdx.x;
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += 64) {
+    const float v = part_val[seq * chunks + c];
+    const int i = part_idx[seq * chunks + c];
+    if (v > best || (v == best && i < best_i)) {
+      best = v;
+      best_i = i;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(best_i, o, 64);
+    if (ov > best || (ov == best && oi < best_i)) {
+      best = ov;
+      best_i = oi;
+    }
+  }
+  if (threadIdx.x == 0) {
+    if (best_i == 0x7fffffff) best_i = 0;  // every token disallowed: torch's argmax of equal -inf is 0
+    out_tokens[seq] = best_i;
+    if (out_logits) out_logits[seq] = best;
+  }
+}
+
 int round_threads(int64_t n, int cap) {
   int64_t t = ((n + 63) / 64) * 64;
   if (t < 64) t = 64;
@@ -266,6 +482,27 @@ void rotary_impl(const hipattn_tensor *positions, hipattn_tensor *query, hipattn
   hipStream_t stream = resolve_stream(stream_arg);
   const int threads = round_threads((int64_t)(Hq + Hkv) * rot_dim / 2, 512);
   const int64_t max_pos = cos_sin->sizes[0];
+  auto a16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (is_neox && dtype_size(query->dtype) == 2 && rot_dim % 16 == 0 && head_size % 8 == 0 &&
+      query->strides[0] % 8 == 0 && key->strides[0] % 8 == 0 && a16(query->data) && a16(key->data) &&
+      a16(cos_sin->data)) {
+    const int vthreads = round_threads((int64_t)(Hq + Hkv) * rot_dim / 16, 512);
+#define HA_ROTV(TT, PP)                                                                                       \
+  rotary_neox_vec8_kernel<TT, PP><<<dim3((unsigned)T), vthreads, 0, stream>>>(                                 \
+      static_cast<const PP *>(positions->data), static_cast<TT *>(query->data), static_cast<TT *>(key->data), \
+      static_cast<const TT *>(cos_sin->data), rot_dim, query->strides[0], key->strides[0], Hq, Hkv, head_size, \
+      max_pos)
+    if (query->dtype == HIPATTN_F16) {
+      if (positions->dtype == HIPATTN_I64) HA_ROTV(half_t, int64_t);
+      else HA_ROTV(half_t, int32_t);
+    } else {
+      if (positions->dtype == HIPATTN_I64) HA_ROTV(bf16_t, int64_t);
+      else HA_ROTV(bf16_t, int32_t);
+    }
+#undef HA_ROTV
+    check_launch("rotary_embedding");
+    return;
+  }
 #define HA_ROT(TT, PP, NX)                                                                              \
   rotary_kernel<TT, PP, NX><<<dim3((unsigned)T), threads, 0, stream>>>(                                  \
       static_cast<const PP *>(positions->data), static_cast<TT *>(query->data), static_cast<TT *>(key->data), \
@@ -311,6 +548,28 @@ void rms_norm_impl(hipattn_tensor *out, hipattn_tensor *input, hipattn_tensor *r
   check_data(other, fused ? "residual" : "out");
   check_data(weight, "weight");
   hipStream_t stream = resolve_stream(stream_arg);
+  auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (dtype_size(input->dtype) == 2 && hidden % 8 == 0 && hidden <= 8192 && al16(input->data) &&
+      al16(other->data) && al16(weight->data)) {
+    const int vthreads = round_threads(hidden / 8, 1024);
+#define HA_RMSV(TT)                                                                                         \
+  if (fused)                                                                                                \
+    rms_norm_vec8_kernel<TT, true><<<dim3((unsigned)rows), vthreads, 0, stream>>>(                           \
+        nullptr, static_cast<TT *>(input->data), static_cast<TT *>(residual->data),                         \
+        static_cast<const TT *>(weight->data), eps, (int)hidden);                                           \
+  else                                                                                                      \
+    rms_norm_vec8_kernel<TT, false><<<dim3((unsigned)rows), vthreads, 0, stream>>>(                          \
+        static_cast<TT *>(out->data), static_cast<TT *>(input->data), nullptr,                              \
+        static_cast<const TT *>(weight->data), eps, (int)hidden)
+    if (input->dtype == HIPATTN_F16) {
+      HA_RMSV(half_t);
+    } else {
+      HA_RMSV(bf16_t);
+    }
+#undef HA_RMSV
+    check_launch(op);
+    return;
+  }
   const int threads = round_threads(hidden, 1024);
 #define HA_RMS(TT)                                                                                          \
   if (fused)                                                                                                \
@@ -349,6 +608,18 @@ void activation_impl(hipattn_tensor *out, const hipattn_tensor *input, int kind,
   check_data(input, "input");
   check_data(out, "out");
   hipStream_t stream = resolve_stream(stream_arg);
+  if (kind == 0 && dtype_size(input->dtype) == 2 && d % 8 == 0 && rows <= 65535 &&
+      (reinterpret_cast<uintptr_t>(input->data) & 15) == 0 && (reinterpret_cast<uintptr_t>(out->data) & 15) == 0) {
+    const dim3 grid((unsigned)((d / 8 + 255) / 256), (unsigned)rows);
+    if (input->dtype == HIPATTN_F16)
+      silu_and_mul_vec8_kernel<half_t><<<grid, 256, 0, stream>>>(static_cast<half_t *>(out->data),
+                                                                 static_cast<const half_t *>(input->data), (int)d);
+    else
+      silu_and_mul_vec8_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<bf16_t *>(out->data),
+                                                                 static_cast<const bf16_t *>(input->data), (int)d);
+    check_launch(op);
+    return;
+  }
   const int threads = round_threads(d, 1024);
 #define HA_ACT(TT)                                                                                     \
   if (kind == 0)                                                                                       \
@@ -417,6 +688,42 @@ void bias_argmax_impl(const hipattn_tensor *logits, const hipattn_tensor *bias, 
   const int threads = round_threads(V, 1024);
   const int32_t *rp = rows ? static_cast<const int32_t *>(rows->data) : nullptr;
   float *ol = out_logits ? static_cast<float *>(out_logits->data) : nullptr;
+  // Wide path: 2-byte logits in 16-byte steps, rows cut into slices so that about a thousand workgroups run.
+  const bool wide = dtype_size(logits->dtype) == 2 && V % 8 == 0 && V >= 16384 && S <= 65535 &&
+                    logits->strides[0] % 8 == 0 && (reinterpret_cast<uintptr_t>(logits->data) & 15) == 0 &&
+                    (!bias || (bias->strides[0] % 4 == 0 && (reinterpret_cast<uintptr_t>(bias->data) & 15) == 0));
+  if (wide) {
+    int64_t chunks = (1024 + S - 1) / S;
+    const int64_t max_chunks = V / 4096;
+    if (chunks > max_chunks) chunks = max_chunks;
+    if (chunks < 1) chunks = 1;
+    const int per_slice = (int)((((V + chunks - 1) / chunks) + 7) / 8 * 8);
+    chunks = (V + per_slice - 1) / per_slice;
+    char *ws = static_cast<char *>(library_workspace((size_t)S * chunks * 8, stream));
+    float *pv = reinterpret_cast<float *>(ws);
+    int32_t *pi = reinterpret_cast<int32_t *>(ws + (size_t)S * chunks * 4);
+    const dim3 grid((unsigned)chunks, (unsigned)S);
+#define HA_BAW(TT)                                                                                               \
+  if (bias)                                                                                                     \
+    bias_argmax_slice_kernel<TT, 0><<<grid, 256, 0, stream>>>(                                                   \
+        static_cast<const TT *>(logits->data), logits->strides[0], static_cast<const float *>(bias->data),      \
+        bias->strides[0], nullptr, 0, 0, rp, (int)V, per_slice, pv, pi);                                        \
+  else                                                                                                          \
+    bias_argmax_slice_kernel<TT, 1><<<grid, 256, 0, stream>>>(                                                   \
+        static_cast<const TT *>(logits->data), logits->strides[0], nullptr, 0,                                  \
+        static_cast<const uint8_t *>(mask->data), mask->strides[0], mask->sizes[1], rp, (int)V, per_slice, pv, pi)
+    if (logits->dtype == HIPATTN_F16) {
+      HA_BAW(half_t);
+    } else {
+      HA_BAW(bf16_t);
+    }
+#undef HA_BAW
+    check_launch("bias_argmax");
+    bias_argmax_pick_kernel<<<dim3((unsigned)S), 64, 0, stream>>>(pv, pi, (int)chunks,
+                                                                 static_cast<int32_t *>(out_tokens->data), ol);
+    check_launch("bias_argmax");
+    return;
+  }
 #define HA_BA(TT)                                                                                               \
   if (bias)                                                                                                     \
     bias_argmax_kernel<TT, 0><<<dim3((unsigned)S), threads, 0, stream>>>(                                        \

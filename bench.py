@@ -68,6 +68,69 @@ def cpu_baseline_decode(c_cpu, rows, threads: int) -> dict:
                       "bytes counted as for the GPU (bf16 K/V once per kv head)"}
 
 
+def streaming_leg(dev, stream, steps: int) -> dict:
+    """The HBM-bound helpers of the path at the sizes of the prefill (config 3: 32768 tokens) and of the
+    full decode step (config 5: 128 x 128256 logits): algorithmic bytes / average launch time (HIP events)."""
+    import numpy as np
+    import torch
+
+    from aici_amd import kernels as K
+    from aici_amd import paged
+    from aici_amd import workloads as W
+    from aici_amd.attn import RotaryEmbedding
+
+    bf = torch.bfloat16
+    res = {}
+
+    def run(name, fn, nbytes):
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        ms = event_times_ms(fn, steps, stream)
+        ms = sum(ms) / len(ms)
+        res[name] = {"us": round(ms * 1e3, 2), "bytes": int(nbytes), "gbs": round(nbytes / ms / 1e6, 1),
+                     "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+    T, H, d, nb = 32768, 8, 128, 2304
+    k = torch.randn(T, H, d, device=dev, dtype=bf)
+    v = torch.randn(T, H, d, device=dev, dtype=bf)
+    kc, vc = paged.alloc_gpu_cache_layer(nb, H, d, 16, bf, dev)
+    blocks = torch.randperm(nb, device=dev)[:T // 16]
+    slots = (blocks.repeat_interleave(16) * 16 + torch.arange(T, device=dev) % 16).to(torch.int64)
+    run("reshape_and_cache 32768 tok x 8 kv heads x 128", lambda: K.reshape_and_cache(k, v, kc, vc, slots),
+        2 * 2 * T * H * d * 2 + 8 * T)
+    s32 = slots.to(torch.int32)
+    ko, vo = torch.empty_like(k), torch.empty_like(v)
+    run("gather_cached_kv 32768 tok x 8 kv heads x 128", lambda: K.gather_cached_kv(ko, vo, kc, vc, s32),
+        2 * 2 * T * H * d * 2 + 4 * T)
+    q2 = torch.randn(T, 32 * 128, device=dev, dtype=bf)
+    k2 = torch.randn(T, 8 * 128, device=dev, dtype=bf)
+    pos = torch.arange(T, device=dev, dtype=torch.int64) % 4096
+    cs = RotaryEmbedding.build_table(128, 500000.0, 4096, bf).to(dev)
+    run("rotary_embedding 32768 tok, 32+8 heads x 128", lambda: K.rotary_embedding(pos, q2, k2, 128, cs, True),
+        2 * T * (32 + 8) * 128 * 2)
+    x = torch.randn(T, 4096, device=dev, dtype=bf)
+    w = torch.randn(4096, device=dev, dtype=bf)
+    o = torch.empty_like(x)
+    run("rms_norm 32768 x 4096", lambda: K.rms_norm(o, x, w, 1e-5), 2 * T * 4096 * 2)
+    r = torch.randn(T, 4096, device=dev, dtype=bf)
+    run("fused_add_rms_norm 32768 x 4096", lambda: K.fused_add_rms_norm(x, r, w, 1e-5), 4 * T * 4096 * 2)
+    gu = torch.randn(T, 2 * 14336, device=dev, dtype=bf)
+    act = torch.empty(T, 14336, device=dev, dtype=bf)
+    run("silu_and_mul 32768 x 14336", lambda: K.silu_and_mul(act, gu), 3 * T * 14336 * 2)
+    del k, v, kc, vc, ko, vo, q2, k2, x, o, r, gu, act
+    S, V = 128, 128256
+    lg = torch.randn(S, V, device=dev, dtype=bf)
+    allowed = W.allow_mask(5, S, V)
+    mask = torch.from_numpy(np.packbits(np.pad(allowed, ((0, 0), (0, (-V) % 32))), axis=1, bitorder="little")).to(dev)
+    run("bias_argmax 128 x 128256, packed allow-bits", lambda: K.bias_argmax(lg, mask=mask), S * V * 2 + mask.numel())
+    row = (V + 1000) & ~63
+    bias = torch.full((S, row), float("-inf"), dtype=torch.float32, device=dev)
+    bias[:, :V][torch.from_numpy(allowed).to(dev)] = 0.0
+    run("bias_argmax 128 x 128256, f32 bias rows", lambda: K.bias_argmax(lg, bias=bias), S * V * 2 + S * V * 4)
+    return res
+
+
 def llama_step_leg(dev, stream, steps: int, layers: int, share_cache: bool) -> dict:
     """One full engine step of a Llama-3-8B-shaped model (random weights): 128 sequences decoding
     one token each over contexts U[1024,16384] (seed 5), every layer with its own paged KV cache,
@@ -140,6 +203,9 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--kv-pools", type=int, default=3, help="copies of the KV pool cycled through by the decode leg")
+    ap.add_argument("--streaming", action="store_true",
+                    help="also time the HBM-bound helper kernels (cache scatter/gather, rotary, norms, "
+                         "activation, bias + arg-max) against the HBM roofline")
     ap.add_argument("--llama-step", action="store_true",
                     help="also time a full Llama-3-8B-shaped decode step with the AICI mask + greedy stage "
                          "(allocates about 170 GB of HBM)")
@@ -248,6 +314,10 @@ def main() -> None:
                          "kernel": "prefill_varlen_kernel, HIP events"},
         }
         del p
+
+    # ---- optional: the streaming helpers -------------------------------------------------------------
+    if args.streaming:
+        line["streaming"] = streaming_leg(dev, stream, max(20, min(args.steps, 100)))
 
     # ---- optional: the full engine step the decode kernel sits in ---------------------------------
     if args.llama_step:

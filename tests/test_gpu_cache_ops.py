@@ -56,6 +56,61 @@ def test_reshape_and_cache_and_gather_bit_exact(device, dtype, slot_dtype, strid
     assert torch.equal(bits(ko), bits(key[valid])) and torch.equal(bits(vo), bits(value[valid]))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("strided", [False, True])
+def test_long_inputs_runs_of_tokens_mixed_with_everything_else(device, dtype, strided):
+    """More than 1024 tokens: the kernels move aligned runs of 8 tokens as tiles and fall back per
+    token elsewhere.  The slot list mixes prompts that fill permuted blocks in order (lengths not
+    multiples of 8, so runs straddle sequences), a prompt that starts in the middle of a block,
+    padding slots inside a run, decode-like random slots, a slot past the cache and a ragged tail."""
+    g = torch.Generator().manual_seed(7)
+    H, d, bs, nb = 4, 96, 16, 200
+    perm = torch.randperm(nb, generator=g).tolist()
+    slots = []
+
+    def prompt(n, start_off=0):
+        need = (start_off + n + bs - 1) // bs
+        blocks = [perm.pop() for _ in range(need)]
+        slots.extend(blocks[(start_off + t) // bs] * bs + (start_off + t) % bs for t in range(n))
+
+    prompt(512)
+    prompt(203)
+    prompt(77, start_off=5)
+    prompt(256)
+    free = [b * bs + o for b in perm[:20] for o in range(bs)]
+    pick = torch.randperm(len(free), generator=g)[:150].tolist()
+    slots.extend(free[i] for i in pick)              # decode-like: unrelated slots
+    del perm[:20]
+    prompt(131)
+    slots[40] = -1                                   # padding inside a run
+    slots[520] = nb * bs + 3                         # outside the cache: dropped
+    T = len(slots)
+    assert T >= 1024 and T % 8 != 0
+    slots_t = torch.tensor(slots, dtype=torch.int64)
+    if strided:
+        qkv = torch.randn((T, 3, H, d), generator=g).to(dtype)
+        key, value = qkv[:, 1], qkv[:, 2]
+    else:
+        key = torch.randn((T, H, d), generator=g).to(dtype)
+        value = torch.randn((T, H, d), generator=g).to(dtype)
+    kc, vc = make_cache(nb, H, d, bs, dtype, fill=-3.0)
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    ok = (slots_t >= 0) & (slots_t < nb * bs)
+    ref.reshape_and_cache(key[ok], value[ok], kc_ref, vc_ref, slots_t[ok])
+    kd, vd = kc.to(device), vc.to(device)
+    src = qkv.to(device) if strided else None
+    key_d, value_d = (src[:, 1], src[:, 2]) if strided else (key.to(device), value.to(device))
+    K.reshape_and_cache(key_d, value_d, kd, vd, slots_t.to(device))
+    assert torch.equal(bits(kd), bits(kc_ref)) and torch.equal(bits(vd), bits(vc_ref))
+    # gather through the same list (invalid slots leave their output rows untouched)
+    ko = torch.full((T, H, d), 9.0, dtype=dtype, device=device)
+    vo = torch.full_like(ko, 9.0)
+    K.gather_cached_kv(ko, vo, kd, vd, slots_t.to(torch.int32).to(device))
+    want_k, want_v = key.clone(), value.clone()
+    want_k[~ok], want_v[~ok] = 9.0, 9.0
+    assert torch.equal(bits(ko), bits(want_k)) and torch.equal(bits(vo), bits(want_v))
+
+
 def test_config1_scatter_bit_exact(device):
     p, extra = W.config1()
     nb = extra["pool_blocks"]

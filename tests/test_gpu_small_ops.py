@@ -105,6 +105,14 @@ def test_activations(device, dtype):
         assert torch.allclose(out.cpu(), want, **tol)
     else:
         assert ulp_diff16(out, want) <= 1
+    # a width the 16-byte kernel takes (multiple of 8), Llama-3-8B's FFN size
+    xw = (torch.randn((3, 2 * 14336), generator=g) * 2).to(dtype)
+    outw = torch.empty((3, 14336), dtype=dtype, device=device)
+    K.silu_and_mul(outw, xw.to(device))
+    if tol:
+        assert torch.allclose(outw.cpu(), ref.silu_and_mul(xw), **tol)
+    else:
+        assert ulp_diff16(outw, ref.silu_and_mul(xw)) <= 1
     for fn, rf in ((K.gelu_new, ref.gelu_new), (K.gelu_fast, ref.gelu_fast)):
         o = torch.empty_like(x).to(device)
         fn(o, x.to(device))
@@ -143,6 +151,15 @@ def test_bias_argmax_bias_rows_and_packed_mask(device, dtype):
     # ties resolve to the lowest token id
     flat = torch.zeros((2, 1000), dtype=dtype, device=device)
     assert K.bias_argmax(flat, bias=torch.zeros((2, 1024), device=device)).tolist() == [0, 0]
+    # ... also across the slices a long row is cut into: equal maxima at ids 70000 and 16, fp16
+    wide = torch.full((3, 131072), -1.0, dtype=torch.float16, device=device)
+    wide[0, 70000] = 2.0
+    wide[0, 16] = 2.0
+    wide[1, 131071] = 5.0
+    allow_all = torch.full((3, 131072 // 8), 255, dtype=torch.uint8, device=device)
+    assert K.bias_argmax(wide, mask=allow_all).tolist() == [16, 131071, 0]
+    allow_all[0, 2] = 0              # forbid ids 16..23: the later maximum wins
+    assert K.bias_argmax(wide, mask=allow_all).tolist() == [70000, 131071, 0]
     with pytest.raises(HipAttnError, match="exactly one"):
         K.bias_argmax(ld)
 
