@@ -108,6 +108,7 @@ _ERR_FUNCS = {
     "hipattn_shutdown": [],
     "hipattn_block_allocator_new": [c_int64, c_int64, POINTER(c_void_p)],
     "hipattn_block_allocator_alloc_seq": [c_void_p, c_int64, c_int64],
+    "hipattn_block_allocator_set_watermark": [c_void_p, ctypes.c_float],
     "hipattn_block_allocator_append_slots": [c_void_p, c_int64, c_int64, c_int64, POINTER(c_int64), c_int64,
                                              POINTER(c_int64)],
     "hipattn_block_allocator_copy": [c_void_p, c_int64, c_int64, c_int64],
@@ -129,6 +130,8 @@ _PLAIN_FUNCS = {
     "hipattn_version": (c_char_p, []),
     "hipattn_block_allocator_free": (None, [c_void_p]),
     "hipattn_block_allocator_num_free": (c_int64, [c_void_p]),
+    "hipattn_block_allocator_can_allocate": (ctypes.c_int, [c_void_p, c_int64]),
+    "hipattn_block_allocator_can_append_slot": (ctypes.c_int, [c_void_p, c_int64]),
     "hipattn_block_allocator_num_allocated": (c_int64, [c_void_p, c_int64]),
     "hipattn_batch_builder_free": (None, [c_void_p]),
     "hipattn_cache_x": (c_int64, [c_int32]),

@@ -13,6 +13,7 @@ struct hipattn_block_allocator {
   int64_t block_size;
   std::vector<int64_t> free_list;   // popped from the back
   std::vector<int64_t> ref_count;   // per physical block
+  int64_t watermark_blocks = 0;     // blocks.rs:262
   std::unordered_map<int64_t, std::vector<int64_t>> seq_blocks;
 
   int64_t num_blocks_for(int64_t length) const { return (length + block_size - 1) / block_size; }
@@ -85,6 +86,24 @@ extern "C" void hipattn_block_allocator_free(hipattn_block_allocator *a) { delet
 
 extern "C" int64_t hipattn_block_allocator_num_free(const hipattn_block_allocator *a) {
   return a ? (int64_t)a->free_list.size() : 0;
+}
+
+extern "C" char *hipattn_block_allocator_set_watermark(hipattn_block_allocator *a, float watermark) {
+  HA_PROTECT({
+    HA_CHECK(a != nullptr, "null allocator");
+    HA_CHECK(watermark >= 0.0f, "watermark must be non-negative");  // blocks.rs:327
+    a->watermark_blocks = (int64_t)(watermark * (float)a->ref_count.size());  // :328, f32 arithmetic, truncated
+  });
+}
+
+extern "C" int hipattn_block_allocator_can_allocate(const hipattn_block_allocator *a, int64_t seq_len) {
+  if (!a || seq_len < 0) return 0;
+  return (int64_t)a->free_list.size() >= a->num_blocks_for(seq_len) + a->watermark_blocks;  // :267-270, :318
+}
+
+extern "C" int hipattn_block_allocator_can_append_slot(const hipattn_block_allocator *a, int64_t num_running_seqs) {
+  if (!a || num_running_seqs < 0) return 0;
+  return (int64_t)a->free_list.size() >= num_running_seqs;  // :278-282
 }
 
 extern "C" int64_t hipattn_block_allocator_num_allocated(const hipattn_block_allocator *a, int64_t seq_id) {

@@ -38,6 +38,18 @@ class BlockAllocator:
     def num_allocated_blocks(self, seq_id: int) -> int:
         return int(_lib.load().hipattn_block_allocator_num_allocated(self._h, int(seq_id)))
 
+    def set_watermark(self, watermark: float) -> None:
+        """blocks.rs:321-343: hold back `watermark * num_blocks` (truncated) blocks from new sequences."""
+        call("hipattn_block_allocator_set_watermark", self._h, float(watermark))
+
+    def can_allocate(self, seq_len: int) -> bool:
+        """blocks.rs:267-270."""
+        return bool(_lib.load().hipattn_block_allocator_can_allocate(self._h, int(seq_len)))
+
+    def can_append_slot(self, num_running_seqs: int) -> bool:
+        """blocks.rs:278-282."""
+        return bool(_lib.load().hipattn_block_allocator_can_append_slot(self._h, int(num_running_seqs)))
+
     def alloc_seq(self, seq_id: int, seq_len: int) -> None:
         call("hipattn_block_allocator_alloc_seq", self._h, int(seq_id), int(seq_len))
 

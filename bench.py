@@ -25,7 +25,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per decode launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB
 # copy (profiles/decode_c2_hbm_traffic.md); bench.py cannot read counters itself.
-DECODE_TRAFFIC_BYTES = 641.0e6
+DECODE_TRAFFIC_BYTES = 643.2e6
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
 
 
@@ -278,7 +278,7 @@ def main() -> None:
                    "context_tokens": int(c_cpu.context_lens.sum()), "kv_pool_copies": len(pools)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": DECODE_TRAFFIC_BYTES,
-                     "kernel": "paged_decode_kernel (+ reduce) per step, HIP events",
+                     "kernel": "paged_decode_flat_kernel + its reduce kernel per step, HIP events on the launch stream",
                      "avg_launch_us": round(avg_launch_ms * 1e3, 2)},
     }
 
@@ -311,7 +311,7 @@ def main() -> None:
                        "algorithmic_flops_per_step": p.flops()},
             "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                         "kernel": "prefill_varlen_kernel, HIP events"},
+                         "kernel": "prefill_varlen_w8_kernel, HIP events on the launch stream"},
         }
         del p
 

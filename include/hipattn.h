@@ -319,6 +319,19 @@ char *hipattn_block_allocator_get_block_idxes(const hipattn_block_allocator *a,
                                               int64_t seq_id, int64_t len,
                                               int64_t *out_slots);
 
+/* Admission policy of `BlockSpaceManager` over the GPU allocator
+ * (blocks.rs:260-283, 321-343): `watermark_blocks = (watermark * num_blocks) as
+ * usize` blocks are held back from new sequences so that running ones can keep
+ * growing.  can_allocate: a new sequence of seq_len tokens fits on top of the
+ * watermark (`can_allocate`, :267-270); can_append_slot: one free block per
+ * running sequence (`can_append_slot`, :278-282).  Both return 0 / 1. */
+char *hipattn_block_allocator_set_watermark(hipattn_block_allocator *a,
+                                            float watermark);
+int hipattn_block_allocator_can_allocate(const hipattn_block_allocator *a,
+                                         int64_t seq_len);
+int hipattn_block_allocator_can_append_slot(const hipattn_block_allocator *a,
+                                            int64_t num_running_seqs);
+
 typedef struct hipattn_batch_builder hipattn_batch_builder;
 
 /* What `BatchInfoBuilder::finish` produces (batch_info.rs:18-43,196-315).  All

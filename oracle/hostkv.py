@@ -45,6 +45,17 @@ class BlockAllocator:
         self.ref_count[idx] += 1
         return idx
 
+    def set_watermark(self, watermark: float) -> None:           # blocks.rs:321-343
+        assert watermark >= 0.0
+        import numpy as np
+        self.watermark_blocks = int(np.float32(watermark) * np.float32(len(self.ref_count)))
+
+    def can_allocate(self, seq_len: int) -> bool:                # blocks.rs:267-270, 318
+        return self.get_num_free_blocks() >= self.num_blocks(seq_len) + getattr(self, "watermark_blocks", 0)
+
+    def can_append_slot(self, num_running_seqs: int) -> bool:    # blocks.rs:278-282
+        return self.get_num_free_blocks() >= num_running_seqs
+
     def get_num_free_blocks(self) -> int:
         return len(self.free_list)
 

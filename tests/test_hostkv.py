@@ -55,6 +55,21 @@ def test_exhaustion_is_an_error_and_leaves_state_unchanged():
         a.get_block_idxes(99, 1)
 
 
+def test_admission_policy_hand_case():
+    """blocks.rs:260-283, 321-343: 1 % of 250 blocks = 2.5 -> 2 blocks held back from new sequences."""
+    for A in (paged.BlockAllocator, ref.BlockAllocator):
+        a = A(16, 250)
+        assert a.can_allocate(250 * 16) and not a.can_allocate(250 * 16 + 1)
+        a.set_watermark(0.01)
+        assert a.can_allocate(248 * 16) and not a.can_allocate(248 * 16 + 1)
+        a.alloc_seq(1, 240 * 16)                      # 10 blocks left, 2 of them held back
+        assert a.can_allocate(8 * 16) and not a.can_allocate(8 * 16 + 1)
+        assert a.can_allocate(0)
+        assert a.can_append_slot(10) and not a.can_append_slot(11)   # appends ignore the watermark
+        a.set_watermark(0.0)
+        assert a.can_allocate(10 * 16)
+
+
 @pytest.mark.parametrize("seed", range(5))
 def test_allocator_random_walk_matches_restatement(seed):
     rng = np.random.default_rng(seed)
