@@ -667,6 +667,41 @@ __global__ __launch_bounds__(128) void paged_decode_flat_reduce_kernel(DecodePar
   const int first_odd = u0 > split.start(w0) ? 1 : 0;
   // slot of piece i: wavefront w0 + i; only the first piece can start inside its wavefront's range
   auto slot = [&](int i) -> int64_t { return (int64_t)(2 * (w0 + i) + (i == 0 ? first_odd : 0)) * p.flat_cols + col; };
+  if (np <= 64) {
+    // Lane i owns piece i's (max, sum); the first pieces' accumulator values are
+    // requested before anything depends on them, so the kernel is two memory
+    // round trips deep (prefix, then everything else).
+    constexpr int NPRE = 8;
+    const int d0 = threadIdx.x;
+    float pre[NPRE];
+#pragma unroll
+    for (int i = 0; i < NPRE; i++) pre[i] = (i < np && d0 < HD) ? p.ws_acc[slot(i) * HD + d0] : 0.f;
+    const float mi = lane < np ? p.ws_m[slot(lane)] : -INFINITY;
+    const float li = lane < np ? p.ws_l[slot(lane)] : 0.f;
+    float mmax = mi;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mmax = fmaxf(mmax, __shfl_xor(mmax, o, 64));
+    const float wi = lane < np ? fast_exp2(mi - mmax) : 0.f;
+    float denom = li * wi;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) denom += __shfl_xor(denom, o, 64);
+    const float inv = denom > 0.f ? 1.0f / denom : 0.f;
+    __shared__ float s_w[64];  // every wavefront computed the same weights; the first one publishes them
+    if (threadIdx.x < 64) s_w[lane] = wi;
+    __syncthreads();
+    for (int d = d0; d < HD; d += blockDim.x) {
+      float o = 0.f;
+      if (d == d0) {
+#pragma unroll
+        for (int i = 0; i < NPRE; i++) o += pre[i] * s_w[i];
+      } else {
+        for (int i = 0; i < NPRE && i < np; i++) o += p.ws_acc[slot(i) * HD + d] * s_w[i];
+      }
+      for (int i = NPRE; i < np; i++) o += p.ws_acc[slot(i) * HD + d] * s_w[i];
+      op[d] = from_float<T>(o * inv);
+    }
+    return;
+  }
   float mmax = -INFINITY;
   for (int i = lane; i < np; i += 64) mmax = fmaxf(mmax, p.ws_m[slot(i)]);
 #pragma unroll
