@@ -759,6 +759,11 @@ void launch_decode_flat(DecodeParams p, int64_t S, int max_context_len, hipStrea
   p.ws_l = p.ws_m + slots;
   paged_decode_flat_kernel<T, HD><<<dim3((unsigned)wgs), 256, 0, stream>>>(p);
   check_launch("paged_attention");
+  // Measurement aid: HIPATTN_DECODE_NO_REDUCE=1 leaves the merge of the partials out, so that events around a
+  // call time the streaming kernel alone (the output is then incomplete).
+  if (const char *e = getenv("HIPATTN_DECODE_NO_REDUCE")) {
+    if (atoi(e) != 0) return;
+  }
   paged_decode_flat_reduce_kernel<T, HD><<<dim3((unsigned)p.Hq, (unsigned)S), HD <= 64 ? 64 : 128, 0, stream>>>(p);
   check_launch("paged_attention reduce");
 }
