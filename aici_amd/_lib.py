@@ -62,6 +62,10 @@ class BatchInfo(ctypes.Structure):
         ("paged_context_lens", POINTER(c_int32)),
         ("paged_block_size", c_int64),
         ("paged_max_context_len", c_int64),
+        ("multi_tables_valid", c_int32),
+        ("multi_max_blocks", c_int64),
+        ("multi_block_tables", POINTER(c_int32)),
+        ("multi_context_lens", POINTER(c_int32)),
     ]
 
 
@@ -72,6 +76,7 @@ ERR = c_void_p  # char* that we must free ourselves
 _ERR_FUNCS = {
     "hipattn_mha_varlen_fwd": [TP, TP, TP, TP, TP, TP, c_int, c_int, c_float, c_float, c_bool, c_bool, c_int, c_int,
                                TP, TP, c_void_p],
+    "hipattn_mha_varlen_fwd_paged": [TP, TP, TP, TP, TP, TP, c_int, c_int, c_float, c_bool, TP, TP, c_void_p],
     "hipattn_paged_attention_v1": [TP, TP, TP, TP, c_int, c_float, TP, TP, c_int, c_int, TP, c_void_p],
     "hipattn_paged_attention_v2": [TP, TP, TP, TP, TP, TP, TP, c_int, c_float, TP, TP, c_int, c_int, TP, c_void_p],
     "hipattn_reshape_and_cache": [TP, TP, TP, TP, TP, c_void_p],
@@ -122,6 +127,8 @@ _ERR_FUNCS = {
     "hipattn_batch_builder_finish": [c_void_p, POINTER(BatchInfo)],
     "hipattn_varlen_attn": [TP, TP, TP, TP, TP, TP, TP, TP, TP, c_int64, c_int, c_int, TP, TP, c_int, c_int, c_float,
                             TP, TP, TP, c_void_p],
+    "hipattn_varlen_attn_paged": [TP, TP, TP, TP, TP, TP, TP, TP, TP, c_int64, c_int, c_int, TP, TP, c_int, c_int,
+                                  c_float, TP, c_void_p],
 }
 
 # name -> (restype, argtypes) for the few calls that do not return an error string.

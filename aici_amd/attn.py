@@ -58,16 +58,35 @@ class RmsNorm:
 
 
 def varlen_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch_info: BatchInfo, key_cache: torch.Tensor,
-                value_cache: torch.Tensor, softmax_scale: Optional[float] = None) -> torch.Tensor:
+                value_cache: torch.Tensor, softmax_scale: Optional[float] = None,
+                paged_prefill: bool = False) -> torch.Tensor:
     """mod.rs:318-354: q [T,Hq,d], k/v [T,Hkv,d] -> [T, Hq*d].
 
     batch_info must already live on the GPU.  The whole composition (scatter,
-    gather, varlen prefill rows, paged decode rows) is one C-ABI call."""
+    gather, varlen prefill rows, paged decode rows) is one C-ABI call.  With
+    `paged_prefill` the multi-token rows read their context from the cache
+    through block tables instead of a gathered copy (needs the builder's
+    multi_block_tables and d <= 128)."""
     T, Hq, d = q.shape
     Hkv = k.size(1)
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
     y = torch.empty((T, Hq, d), dtype=q.dtype, device=q.device)
+    if paged_prefill:
+        if batch_info.multi_block_tables is None:
+            raise ValueError("paged_prefill needs batch_info.multi_block_tables (slots must follow the blocks in order)")
+        has_m, has_p = batch_info.q_multi > 0, batch_info.q_multi < T
+        call("hipattn_varlen_attn_paged", _desc(q, "q"), _desc(k, "k"), _desc(v, "v"), _desc(key_cache, "key_cache"),
+             _desc(value_cache, "value_cache"), _desc(batch_info.slot_mapping, "slot_mapping"),
+             _desc(batch_info.multi_block_tables, "multi_block_tables") if has_m else None,
+             _desc(batch_info.seqlens_q, "seqlens_q") if has_m else None,
+             _desc(batch_info.multi_context_lens, "multi_context_lens") if has_m else None, int(batch_info.q_multi),
+             int(batch_info.max_seqlen_q), int(batch_info.max_seqlen_k),
+             _desc(batch_info.paged_block_tables, "paged_block_tables") if has_p else None,
+             _desc(batch_info.paged_context_lens, "paged_context_lens") if has_p else None,
+             int(batch_info.paged_block_size), int(batch_info.paged_max_context_len), float(softmax_scale),
+             _desc(y, "y"), _stream(q))
+        return y.reshape(T, Hq * d)
     G = batch_info.gather_mapping.numel()
     gk = torch.empty((G, Hkv, d), dtype=q.dtype, device=q.device) if G else None
     gv = torch.empty_like(gk) if G else None

@@ -69,3 +69,40 @@ extern "C" char *hipattn_varlen_attn(const hipattn_tensor *q, const hipattn_tens
     }
   });
 }
+
+extern "C" char *hipattn_varlen_attn_paged(const hipattn_tensor *q, const hipattn_tensor *k, const hipattn_tensor *v,
+                                           hipattn_tensor *key_cache, hipattn_tensor *value_cache,
+                                           const hipattn_tensor *slot_mapping, const hipattn_tensor *multi_block_tables,
+                                           const hipattn_tensor *seqlens_q, const hipattn_tensor *multi_context_lens,
+                                           int64_t q_multi, int max_seqlen_q, int max_seqlen_k,
+                                           const hipattn_tensor *paged_block_tables,
+                                           const hipattn_tensor *paged_context_lens, int paged_block_size,
+                                           int paged_max_context_len, float softmax_scale, hipattn_tensor *y,
+                                           void *stream) {
+  HA_PROTECT({
+    check_tensor(q, "q", 3);
+    check_tensor(k, "k", 3);
+    check_tensor(v, "v", 3);
+    check_tensor(y, "y", 3);
+    const int64_t T = q->sizes[0];
+    HA_CHECK(k->sizes[0] == T && v->sizes[0] == T && y->sizes[0] == T, "varlen_attn: q, k, v, y disagree on the token count");
+    HA_CHECK(q_multi >= 0 && q_multi <= T, "varlen_attn: q_multi %lld outside [0, %lld]", (long long)q_multi, (long long)T);
+    const int num_kv_heads = (int)k->sizes[1];
+    raise(hipattn_reshape_and_cache(k, v, key_cache, value_cache, slot_mapping, stream));
+    if (q_multi > 0) {
+      HA_CHECK(multi_block_tables && multi_context_lens && seqlens_q,
+               "varlen_attn: multi-token rows need their block tables, context lens and seqlens_q");
+      hipattn_tensor qm = rows(q, 0, q_multi);
+      hipattn_tensor ym = rows(y, 0, q_multi);
+      raise(hipattn_mha_varlen_fwd_paged(&qm, key_cache, value_cache, multi_block_tables, seqlens_q, multi_context_lens,
+                                         max_seqlen_q, max_seqlen_k, softmax_scale, true, &ym, nullptr, stream));
+    }
+    if (q_multi < T) {
+      HA_CHECK(paged_block_tables && paged_context_lens, "varlen_attn: single-token rows need block tables and context lens");
+      hipattn_tensor qs = rows(q, q_multi, T);
+      hipattn_tensor ys = rows(y, q_multi, T);
+      raise(hipattn_paged_attention_v1(&ys, &qs, key_cache, value_cache, num_kv_heads, softmax_scale, paged_block_tables,
+                                       paged_context_lens, paged_block_size, paged_max_context_len, nullptr, stream));
+    }
+  });
+}

@@ -63,6 +63,7 @@ struct hipattn_batch_builder {
   // outputs of the last finish()
   std::vector<int32_t> tokens, slot_mapping, logit_idxs, seqlens_q, seqlens_k, gather_mapping, tables, ctx_lens;
   std::vector<int64_t> positions, seq_ids;
+  std::vector<int32_t> multi_tables, multi_ctx_lens;
 };
 
 using namespace hipattn;
@@ -286,6 +287,7 @@ extern "C" char *hipattn_batch_builder_finish(hipattn_batch_builder *b, hipattn_
     typedef hipattn_batch_builder::Entry Entry;
     b->tokens.clear(); b->slot_mapping.clear(); b->logit_idxs.clear(); b->seqlens_q.clear(); b->seqlens_k.clear();
     b->gather_mapping.clear(); b->tables.clear(); b->ctx_lens.clear(); b->positions.clear(); b->seq_ids.clear();
+    b->multi_tables.clear(); b->multi_ctx_lens.clear();
 
     // batch_info.rs:209-223: single-token entries to the back (stable), when
     // the paged kernel is enabled; otherwise everything is "multi".
@@ -297,7 +299,8 @@ extern "C" char *hipattn_batch_builder_finish(hipattn_batch_builder *b, hipattn_
     HA_CHECK(!b->entries.empty(), "batch builder: no entries");  // batch_info.rs:255
 
     std::vector<int64_t> lens_q, lens_k;
-    std::vector<std::vector<int32_t>> tables;
+    std::vector<std::vector<int32_t>> tables, multi_tables;
+    bool multi_valid = true;
     int64_t first_single = 0;
     for (size_t idx = 0; idx < b->entries.size(); idx++) {
       const Entry &e = b->entries[idx];
@@ -316,6 +319,19 @@ extern "C" char *hipattn_batch_builder_finish(hipattn_batch_builder *b, hipattn_
         first_single = (int64_t)b->tokens.size();
         lens_q.push_back((int64_t)e.q_tok.size());
         lens_k.push_back((int64_t)e.kv_slots.size());
+        // block table of the entry, valid when its slots walk its blocks in order
+        std::vector<int32_t> row;
+        for (size_t i = 0; i < e.kv_slots.size(); i++) {
+          const int64_t slot = e.kv_slots[i];
+          if (i % (size_t)b->block_size == 0) {
+            if (slot < 0 || slot % b->block_size != 0) multi_valid = false;
+            row.push_back((int32_t)(slot < 0 ? 0 : slot / b->block_size));
+          } else if (slot != (int64_t)row.back() * b->block_size + (int64_t)(i % (size_t)b->block_size)) {
+            multi_valid = false;
+          }
+        }
+        multi_tables.push_back(std::move(row));
+        b->multi_ctx_lens.push_back((int32_t)e.kv_slots.size());
       } else {
         b->ctx_lens.push_back((int32_t)e.kv_slots.size());
         std::vector<int32_t> row;
@@ -346,6 +362,12 @@ extern "C" char *hipattn_batch_builder_finish(hipattn_batch_builder *b, hipattn_
       r.resize(max_row, 0);
       b->tables.insert(b->tables.end(), r.begin(), r.end());
     }
+    size_t multi_row = 0;
+    for (const auto &r : multi_tables) multi_row = std::max(multi_row, r.size());
+    for (auto &r : multi_tables) {
+      r.resize(multi_row, 0);
+      b->multi_tables.insert(b->multi_tables.end(), r.begin(), r.end());
+    }
     int32_t max_ctx = 0;
     for (int32_t cl : b->ctx_lens) max_ctx = std::max(max_ctx, cl);
 
@@ -371,6 +393,10 @@ extern "C" char *hipattn_batch_builder_finish(hipattn_batch_builder *b, hipattn_
     o.paged_context_lens = b->ctx_lens.data();
     o.paged_block_size = b->block_size;
     o.paged_max_context_len = max_ctx;
+    o.multi_tables_valid = multi_valid ? 1 : 0;
+    o.multi_max_blocks = (int64_t)multi_row;
+    o.multi_block_tables = b->multi_tables.data();
+    o.multi_context_lens = b->multi_ctx_lens.data();
     b->entries.clear();
   });
 }

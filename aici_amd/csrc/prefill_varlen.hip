@@ -76,6 +76,14 @@ struct PrefillParams {
   int n_qblocks;
   float scale_log2;
   int causal;
+  // K/V read straight from the paged cache (prefill_varlen_w8_kernel<..., PAGED = true>): k and v are
+  // the caches, position p of sequence b lives in block block_tables[b][p / 16] at offset p % 16.
+  const int32_t *block_tables;
+  const int32_t *context_lens;  // keys per sequence
+  int64_t table_stride;
+  int table_cols;
+  int64_t num_blocks;
+  int64_t kc_block, kc_head, vc_block, vc_head;  // cache strides in elements
 };
 
 template <typename T>
@@ -415,7 +423,7 @@ struct TileW8 {
   static constexpr size_t LDS_BYTES = 3 * (size_t)STAGE_ELEMS * 2;
 };
 
-template <typename T, int HDP>
+template <typename T, int HDP, bool PAGED>
 __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams p) {
   typedef typename Vec8<T>::type vec8;
   typedef TileW8<HDP> TL;
@@ -448,9 +456,9 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
 
   const int q_begin = p.cu_q[b];
   const int Lq = p.cu_q[b + 1] - q_begin;
-  const int k_begin = p.cu_k[b];
-  int Lk = p.cu_k[b + 1] - k_begin;
-  if (p.seqused_k) Lk = min(Lk, p.seqused_k[b]);
+  const int k_begin = PAGED ? 0 : p.cu_k[b];
+  int Lk = PAGED ? p.context_lens[b] : p.cu_k[b + 1] - k_begin;
+  if (!PAGED && p.seqused_k) Lk = min(Lk, p.seqused_k[b]);
   const int wg_row0 = qb * BM;
   if (wg_row0 >= Lq) return;
   const int off = Lk - Lq;
@@ -462,8 +470,8 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   const int wave_last_row = wave_row0 + 31;
 
   const T *qp = static_cast<const T *>(p.q) + (int64_t)q_begin * p.q_row + (int64_t)h * p.q_head;
-  const T *kp = static_cast<const T *>(p.k) + (int64_t)k_begin * p.k_row + (int64_t)kvh * p.k_head;
-  const T *vp = static_cast<const T *>(p.v) + (int64_t)k_begin * p.v_row + (int64_t)kvh * p.v_head;
+  const T *kp = static_cast<const T *>(p.k) + (PAGED ? (int64_t)kvh * p.kc_head : (int64_t)k_begin * p.k_row + (int64_t)kvh * p.k_head);
+  const T *vp = static_cast<const T *>(p.v) + (PAGED ? (int64_t)kvh * p.vc_head : (int64_t)k_begin * p.v_row + (int64_t)kvh * p.v_head);
   const int d_chunks = p.d / 8;
 
   vec8 qreg[KSTEPS];
@@ -507,7 +515,47 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     k_boff[i] = (uint32_t)(((int64_t)(idx / CPR) * p.k_row + min(idx % CPR, d_chunks - 1) * 8) * (int64_t)sizeof(T));
   }
   const uint32_t v_boff = (uint32_t)(((int64_t)(v_kg4 * 4) * p.v_row + min(v_dg, p.d / 4 - 1) * 4) * (int64_t)sizeof(T));
-  auto load_tile = [&](int tile) {
+  // PAGED: blocks of the cache instead of rows of k / v.  A tile is 4 blocks; threads follow the cache's
+  // own order so that consecutive lanes read consecutive 16-byte runs: K unit u = (block, chunk c8,
+  // token) is the run [c8][token] of its block and lands in LDS row 16*block + token; V unit u = (block,
+  // head element, half) is 8 tokens of the cache's [d][token] row -- already transposed.
+  constexpr int K_PER_BLOCK = CPR * 16;            // 16-byte K runs per block
+  constexpr int V_PER_BLOCK = HDP * 2;             // 16-byte V runs per block
+  constexpr int NLOADVP = (4 * V_PER_BLOCK + 511) / 512;
+  u32x4_t vstp[PAGED ? NLOADVP : 1];
+  int staged_k0 = 0;  // first key of the tile held in the staging registers
+  const int32_t *table_row = PAGED ? p.block_tables + (int64_t)b * p.table_stride : nullptr;
+  auto table_block = [&](int col) -> int64_t {
+    const int64_t blk = table_row[min(col, p.table_cols - 1)];
+    return blk < 0 ? 0 : (blk >= p.num_blocks ? p.num_blocks - 1 : blk);
+  };
+  auto load_tile_paged = [&](int tile) {
+    const int k0 = tile * BN;
+    staged_k0 = k0;
+    // Blocks wholly or partly inside the context; a block past it re-reads the last one (its keys are
+    // masked, its V runs cleared before they reach LDS).
+    const int last_col = (Lk - 1) >> 4;
+    int64_t blk[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) blk[r] = table_block(min(k0 / 16 + r, last_col));
+#pragma unroll
+    for (int i = 0; i < NLOADK; i++) {
+      const int u = min(tid + 512 * i, K_CHUNKS - 1);
+      const int r = u / K_PER_BLOCK, rem = u % K_PER_BLOCK;
+      const int c8 = min(rem / 16, d_chunks - 1), tok = rem % 16;
+      const int64_t bs = r == 0 ? blk[0] : (r == 1 ? blk[1] : (r == 2 ? blk[2] : blk[3]));
+      kst[i] = *reinterpret_cast<const u32x4_t *>(kp + bs * p.kc_block + (c8 * 16 + tok) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < NLOADVP; i++) {
+      const int u = min(tid + 512 * i, 4 * V_PER_BLOCK - 1);
+      const int r = u / V_PER_BLOCK, rem = u % V_PER_BLOCK;
+      const int drow = min(rem / 2, p.d - 1), half = rem % 2;
+      const int64_t bs = r == 0 ? blk[0] : (r == 1 ? blk[1] : (r == 2 ? blk[2] : blk[3]));
+      vstp[i] = *reinterpret_cast<const u32x4_t *>(vp + bs * p.vc_block + drow * 16 + half * 8);
+    }
+  };
+  auto load_tile_rows = [&](int tile) {
     const int k0 = tile * BN;
     if (k0 + BN <= Lk) {
       const char *kt = reinterpret_cast<const char *>(kp + (int64_t)k0 * p.k_row);
@@ -531,7 +579,49 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       }
     }
   };
-  auto store_tile = [&](int stage) {
+  auto load_tile = [&](int tile) {
+    if constexpr (PAGED)
+      load_tile_paged(tile);
+    else
+      load_tile_rows(tile);
+  };
+  auto store_tile_paged = [&](int stage) {
+    T *ks = smem + stage * TL::STAGE_ELEMS;
+    T *vs = ks + TL::K_ELEMS;
+#pragma unroll
+    for (int i = 0; i < NLOADK; i++) {
+      const int u = tid + 512 * i;
+      if (K_CHUNKS % 512 == 0 || u < K_CHUNKS) {
+        const int r = u / K_PER_BLOCK, rem = u % K_PER_BLOCK;
+        *reinterpret_cast<u32x4_t *>(ks + (r * 16 + rem % 16) * TL::KSTR + (rem / 16) * 8) = kst[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NLOADVP; i++) {
+      const int u = tid + 512 * i;
+      if ((4 * V_PER_BLOCK) % 512 == 0 || u < 4 * V_PER_BLOCK) {
+        const int r = u / V_PER_BLOCK, rem = u % V_PER_BLOCK;
+        const int drow = rem / 2, half = rem % 2;
+        u32x4_t o = vstp[i];
+        // Cache tokens past the context hold whatever was there before (possibly NaN, which a zero
+        // probability would not neutralise): clear them.
+        if (staged_k0 + BN > Lk) {
+          const int alive = Lk - (staged_k0 + r * 16 + half * 8);  // keys of this run inside the context
+#pragma unroll
+          for (int w = 0; w < 4; w++) {
+            const int a2 = alive - 2 * w;
+            o[w] &= a2 <= 0 ? 0u : (a2 == 1 ? 0xffffu : 0xffffffffu);
+          }
+        }
+        // the run's two groups of 4 keys: groups (2 half, 2 half + 1) of block r -> positions 8 half, 8 half + 4
+        // in the order the MFMA operand wants them: [g(8) a(4) b] from [a(8) g(4) b]
+        T *row = vs + drow * TL::VTSTR + r * 16;
+        *reinterpret_cast<u32x2_t *>(row + half * 4) = u32x2_t{o[0], o[1]};
+        *reinterpret_cast<u32x2_t *>(row + 8 + half * 4) = u32x2_t{o[2], o[3]};
+      }
+    }
+  };
+  auto store_tile_rows = [&](int stage) {
     T *ks = smem + stage * TL::STAGE_ELEMS;
     T *vs = ks + TL::K_ELEMS;
 #pragma unroll
@@ -561,6 +651,12 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
           *reinterpret_cast<u32x2_t *>(vs + (v_dg * 4 + dd) * TL::VTSTR + pos) = o[dd];
       }
     }
+  };
+  auto store_tile = [&](int stage) {
+    if constexpr (PAGED)
+      store_tile_paged(stage);
+    else
+      store_tile_rows(stage);
   };
 
   if (n_tiles > 0) {
@@ -769,10 +865,10 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   }
 }
 
-template <typename T, int HDP>
+template <typename T, int HDP, bool PAGED = false>
 void launch_prefill_w8(PrefillParams p, hipStream_t stream) {
   static bool attr_set = false;  // benign race: setting twice is harmless
-  auto kernel = prefill_varlen_w8_kernel<T, HDP>;
+  auto kernel = prefill_varlen_w8_kernel<T, HDP, PAGED>;
   if (!attr_set) {
     HA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)TileW8<HDP>::LDS_BYTES));
@@ -952,10 +1048,132 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
   else dispatch_hd<bf16_t>(p, total_q, stream);
 }
 
+// Varlen prefill whose keys and values are read from the paged cache through block tables: what
+// rLLM composes from gather_cached_kv -> repeat_kv -> flash_attn_varlen (llm/mod.rs:181-238) without
+// the two copies.  Eight-wavefront kernel only (head sizes up to 128).
+template <typename T>
+void dispatch_paged(const PrefillParams &p, hipStream_t stream) {
+  const int hdp = ((p.d + 31) / 32) * 32;
+  switch (hdp) {
+    case 32: launch_prefill_w8<T, 32, true>(p, stream); break;
+    case 64: launch_prefill_w8<T, 64, true>(p, stream); break;
+    case 96: launch_prefill_w8<T, 96, true>(p, stream); break;
+    case 128: launch_prefill_w8<T, 128, true>(p, stream); break;
+    default: fail("mha_varlen_fwd_paged: head size %d not supported (at most 128)", p.d);
+  }
+}
+
+void mha_varlen_fwd_paged_impl(const hipattn_tensor *q, const hipattn_tensor *key_cache,
+                               const hipattn_tensor *value_cache, const hipattn_tensor *block_tables,
+                               const hipattn_tensor *cu_q, const hipattn_tensor *context_lens, int max_q, int max_k,
+                               float scale, bool causal, hipattn_tensor *out, hipattn_tensor *lse, void *stream_arg) {
+  const char *op = "mha_varlen_fwd_paged";
+  check_tensor(q, "q", 3);
+  HA_CHECK(q->dtype == HIPATTN_F16 || q->dtype == HIPATTN_BF16, "%s: only fp16 and bf16 are supported, got %s", op,
+           dtype_name(q->dtype));
+  const int d = (int)q->sizes[2];
+  const int Hq = (int)q->sizes[1];
+  HA_CHECK(d % 8 == 0 && d > 0 && d <= 128, "%s: head size must be a multiple of 8 in (0, 128], got %d", op, d);
+  check_qkv(q, "q", q->dtype, d);
+  check_qkv(out, "out", q->dtype, d);
+  HA_CHECK(out->sizes[0] == q->sizes[0] && out->sizes[1] == Hq, "%s: out shape differs from q", op);
+  check_tensor(key_cache, "key_cache", 5);
+  check_tensor(value_cache, "value_cache", 4);
+  HA_CHECK(key_cache->dtype == q->dtype && value_cache->dtype == q->dtype, "%s: caches must have q's dtype", op);
+  const int Hkv = (int)key_cache->sizes[1];
+  HA_CHECK(Hkv > 0 && Hq % Hkv == 0, "%s: %d query heads not divisible by %d kv heads", op, Hq, Hkv);
+  HA_CHECK(key_cache->sizes[2] * key_cache->sizes[4] == d && key_cache->sizes[3] == 16 && key_cache->sizes[4] == 8,
+           "%s: key_cache shape does not match [nb, %d, %d/8, 16, 8]", op, Hkv, d);
+  HA_CHECK(value_cache->sizes[0] == key_cache->sizes[0] && value_cache->sizes[1] == Hkv &&
+               value_cache->sizes[2] == d && value_cache->sizes[3] == 16,
+           "%s: value_cache shape does not match [nb, %d, %d, 16]", op, Hkv, d);
+  HA_CHECK(key_cache->strides[4] == 1 && key_cache->strides[3] == 8 && key_cache->strides[2] == 128 &&
+               value_cache->strides[3] == 1 && value_cache->strides[2] == 16,
+           "%s: cache inner dims must be contiguous", op);
+  HA_CHECK(key_cache->strides[0] % 8 == 0 && key_cache->strides[1] % 8 == 0 && value_cache->strides[0] % 4 == 0 &&
+               value_cache->strides[1] % 4 == 0 && (reinterpret_cast<uintptr_t>(key_cache->data) & 15) == 0 &&
+               (reinterpret_cast<uintptr_t>(value_cache->data) & 15) == 0,
+           "%s: caches must be 16-byte aligned", op);
+  HA_CHECK(key_cache->sizes[0] > 0, "%s: the cache has no blocks", op);
+  check_tensor(cu_q, "cu_seqlens_q", 1);
+  check_tensor(context_lens, "context_lens", 1);
+  check_tensor(block_tables, "block_tables", 2);
+  HA_CHECK(cu_q->dtype == HIPATTN_I32 && context_lens->dtype == HIPATTN_I32 && block_tables->dtype == HIPATTN_I32,
+           "%s: cu_seqlens_q, context_lens and block_tables must be int32", op);
+  check_contiguous(cu_q, "cu_seqlens_q");
+  check_contiguous(context_lens, "context_lens");
+  HA_CHECK(cu_q->sizes[0] >= 1, "%s: cu_seqlens_q must hold batch+1 entries", op);
+  const int batch = (int)cu_q->sizes[0] - 1;
+  HA_CHECK(context_lens->sizes[0] == batch && block_tables->sizes[0] == batch,
+           "%s: context_lens and block_tables need %d rows", op, batch);
+  HA_CHECK(block_tables->sizes[1] <= 1 || block_tables->strides[1] == 1, "%s: block_tables rows must be contiguous", op);
+  HA_CHECK(scale > 0.f, "%s: softmax_scale must be positive", op);
+  HA_CHECK(max_q >= 0 && max_k >= 0, "%s: negative max_seqlen", op);
+  HA_CHECK((int64_t)(max_k + 15) / 16 <= block_tables->sizes[1], "%s: max_seqlen_k %d needs more than the %lld block-table columns",
+           op, max_k, (long long)block_tables->sizes[1]);
+  if (lse) {
+    check_tensor(lse, "softmax_lse", 3);
+    HA_CHECK(lse->dtype == HIPATTN_F32 && lse->sizes[0] == batch && lse->sizes[1] == Hq && lse->sizes[2] >= max_q,
+             "%s: softmax_lse must be f32 [batch, Hq, >= max_seqlen_q]", op);
+    check_contiguous(lse, "softmax_lse");
+    check_data(lse, "softmax_lse");
+  }
+  const int64_t total_q = q->sizes[0];
+  if (batch == 0 || total_q == 0 || Hq == 0 || max_q == 0) return;
+  check_data(cu_q, "cu_seqlens_q");
+  check_data(context_lens, "context_lens");
+  check_data(block_tables, "block_tables");
+  check_data(key_cache, "key_cache");
+  check_data(value_cache, "value_cache");
+  hipStream_t stream = resolve_stream(stream_arg);
+
+  PrefillParams p;
+  memset(&p, 0, sizeof p);
+  p.q = q->data;
+  p.k = key_cache->data;
+  p.v = value_cache->data;
+  p.out = out->data;
+  p.lse = lse ? static_cast<float *>(lse->data) : nullptr;
+  p.q_row = q->strides[0];
+  p.q_head = q->strides[1];
+  p.o_row = out->strides[0];
+  p.o_head = out->strides[1];
+  p.cu_q = static_cast<const int32_t *>(cu_q->data);
+  p.batch = batch;
+  p.Hq = Hq;
+  p.Hkv = Hkv;
+  p.G = Hq / Hkv;
+  p.d = d;
+  p.max_q = max_q;
+  p.lse_pitch = lse ? (int)lse->sizes[2] : 0;
+  p.scale_log2 = scale * kLog2e;
+  p.causal = causal ? 1 : 0;
+  p.block_tables = static_cast<const int32_t *>(block_tables->data);
+  p.context_lens = static_cast<const int32_t *>(context_lens->data);
+  p.table_stride = block_tables->strides[0];
+  p.table_cols = (int)block_tables->sizes[1];
+  p.num_blocks = key_cache->sizes[0];
+  p.kc_block = key_cache->strides[0];
+  p.kc_head = key_cache->strides[1];
+  p.vc_block = value_cache->strides[0];
+  p.vc_head = value_cache->strides[1];
+  if (q->dtype == HIPATTN_F16) dispatch_paged<half_t>(p, stream);
+  else dispatch_paged<bf16_t>(p, stream);
+}
+
 }  // namespace
 }  // namespace hipattn
 
 using namespace hipattn;
+
+extern "C" char *hipattn_mha_varlen_fwd_paged(const hipattn_tensor *q, const hipattn_tensor *key_cache,
+                                              const hipattn_tensor *value_cache, const hipattn_tensor *block_tables,
+                                              const hipattn_tensor *cu_seqlens_q, const hipattn_tensor *context_lens,
+                                              int max_seqlen_q, int max_seqlen_k, float softmax_scale, bool is_causal,
+                                              hipattn_tensor *out, hipattn_tensor *softmax_lse, void *stream) {
+  HA_PROTECT(mha_varlen_fwd_paged_impl(q, key_cache, value_cache, block_tables, cu_seqlens_q, context_lens, max_seqlen_q,
+                                       max_seqlen_k, softmax_scale, is_causal, out, softmax_lse, stream));
+}
 
 extern "C" char *hipattn_mha_varlen_fwd(const hipattn_tensor *q, const hipattn_tensor *k, const hipattn_tensor *v,
                                         const hipattn_tensor *cu_seqlens_q, const hipattn_tensor *cu_seqlens_k,

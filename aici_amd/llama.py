@@ -109,8 +109,10 @@ class Llama:
         kernels.rms_norm(out, x, weight, self.cfg.rms_norm_eps)
         return out
 
-    def forward(self, batch_info: BatchInfo, caches: List[Tuple[torch.Tensor, torch.Tensor]]) -> torch.Tensor:
-        """batch_info on the device; caches[layer] = (key_cache, value_cache), updated in place."""
+    def forward(self, batch_info: BatchInfo, caches: List[Tuple[torch.Tensor, torch.Tensor]],
+                paged_prefill: bool = False) -> torch.Tensor:
+        """batch_info on the device; caches[layer] = (key_cache, value_cache), updated in place.
+        paged_prefill: multi-token rows read their context through block tables (no gather copy)."""
         cfg = self.cfg
         Hq, Hkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
         x = self.wte.index_select(0, batch_info.tokens.long())                   # llama.rs:203
@@ -120,7 +122,7 @@ class Llama:
             qkv = h @ layer["qkv"].t()                                          # :81-83
             q, k, v = (t.contiguous() for t in qkv.split([Hq * d, Hkv * d, Hkv * d], dim=1))
             q, k = self.rotary.forward(batch_info.positions, q, k)              # :85 (in place on the copies)
-            y = varlen_attn(q, k, v.reshape(T, Hkv, d), batch_info, kc, vc)     # :93
+            y = varlen_attn(q, k, v.reshape(T, Hkv, d), batch_info, kc, vc, paged_prefill=paged_prefill)  # :93
             x = y @ layer["o"].t() + x                                          # :96, :166
             h = self._rms(x, layer["rms_2"])                                    # :169
             gu = h @ layer["gate_up"].t()                                       # :135-136

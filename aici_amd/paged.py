@@ -97,6 +97,10 @@ class BatchInfo:
     paged_max_context_len: int
     seqlen_multi: int
     q_multi: int
+    # extension: block tables / key counts of the multi-token entries (None when some entry's slots do not
+    # walk its blocks in order, in which case only the gather route applies)
+    multi_block_tables: Optional[torch.Tensor] = None
+    multi_context_lens: Optional[torch.Tensor] = None
 
     def to(self, device) -> "BatchInfo":
         kw = dict(self.__dict__)
@@ -165,6 +169,10 @@ class BatchInfoBuilder:
             paged_max_context_len=int(bi.paged_max_context_len),
             seqlen_multi=nm,
             q_multi=int(bi.q_multi),
+            multi_block_tables=(torch.from_numpy(_np(bi.multi_block_tables, nm * int(bi.multi_max_blocks), np.int32))
+                                .reshape(nm, int(bi.multi_max_blocks)) if bi.multi_tables_valid else None),
+            multi_context_lens=(torch.from_numpy(_np(bi.multi_context_lens, nm, np.int32))
+                                if bi.multi_tables_valid else None),
         )
 
 

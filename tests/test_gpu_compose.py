@@ -16,7 +16,8 @@ from tests.common import TOL, make_cache
 pytestmark = pytest.mark.gpu
 
 
-def mixed_step(seed, chunk_priors, chunk_len, n_decode, ctx_lo, ctx_hi, Hq, Hkv, d, dtype, pool, fused_qkv, device):
+def mixed_step(seed, chunk_priors, chunk_len, n_decode, ctx_lo, ctx_hi, Hq, Hkv, d, dtype, pool, fused_qkv, device,
+               paged_prefill=False):
     rng = np.random.default_rng(seed)
     g = torch.Generator().manual_seed(seed)
     bs = 16
@@ -74,7 +75,7 @@ def mixed_step(seed, chunk_priors, chunk_len, n_decode, ctx_lo, ctx_hi, Hq, Hkv,
         qd, kd_in, vd_in = qkv_d[:, 0], qkv_d[:, 1], qkv_d[:, 2]
     else:
         qd, kd_in, vd_in = q.to(device), k.to(device), v.to(device)
-    y = attn.varlen_attn(qd, kd_in, vd_in, bi.to(device), kd, vd)
+    y = attn.varlen_attn(qd, kd_in, vd_in, bi.to(device), kd, vd, paged_prefill=paged_prefill)
     return y.cpu().reshape(T, Hq, d), want, (kd.cpu(), vd.cpu(), kc_ref, vc_ref), bi
 
 
@@ -95,6 +96,23 @@ def test_mixed_step_phi2_shape_reduced(device, fused_qkv):
 def test_mixed_step_gqa_bf16(device):
     y, want, _, bi = mixed_step(32, [0, 17, 640], 200, 33, 1, 900, 32, 8, 128, torch.bfloat16, 2048, False, device)
     assert (y.float() - want).abs().max().item() <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("case", ["phi2", "gqa", "all_prefill"])
+def test_paged_prefill_route(device, case):
+    """The same steps with the multi-token rows reading the cache through block tables
+    (hipattn_varlen_attn_paged) instead of a gathered copy."""
+    if case == "phi2":
+        args, dtype = (31, [0, 100, 200, 300], 64, 20, 30, 500, 32, 32, 80, torch.float16, 1024, True), torch.float16
+    elif case == "gqa":
+        args, dtype = (32, [0, 17, 640], 200, 33, 1, 900, 32, 8, 128, torch.bfloat16, 2048, False), torch.bfloat16
+    else:
+        args, dtype = (33, [0, 0, 0], 150, 0, 1, 2, 8, 8, 64, torch.float16, 256, False), torch.float16
+    y, want, (kc, vc, kc_ref, vc_ref), bi = mixed_step(*args, device, paged_prefill=True)
+    assert bi.multi_block_tables is not None and bi.multi_context_lens.numel() == bi.seqlen_multi
+    assert not torch.isnan(y.float()).any()
+    assert (y.float() - want).abs().max().item() <= TOL[dtype]
+    assert torch.equal(kc.view(torch.int16), kc_ref.view(torch.int16))
 
 
 def test_all_prefill_and_all_decode_steps(device):

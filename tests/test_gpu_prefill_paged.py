@@ -1,0 +1,120 @@
+"""Varlen prefill that reads K/V from the paged cache through block tables
+(hipattn_mha_varlen_fwd_paged) against the oracle's route for the same rows -- gather_cached_kv,
+repeat_kv, varlen SDPA (llm/mod.rs:181-238 on the CPU build) -- and against the library's own
+gather + flash_attn_varlen.  Same gates as the contiguous prefill."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from aici_amd import kernels as K
+from aici_amd import workloads as W
+from aici_amd._lib import HipAttnError
+from oracle import refkernels as ref
+from tests.common import TOL, make_cache
+
+pytestmark = pytest.mark.gpu
+
+
+def paged_case(seed, seqs, Hq, Hkv, d, dtype, pool):
+    """seqs: (prior, new) token counts.  Every context's K/V (prior and new) is in the cache; every slot no
+    context covers holds NaN, as an uninitialised cache may."""
+    g = torch.Generator().manual_seed(seed)
+    rng = np.random.default_rng(seed)
+    kc, vc = make_cache(pool, Hkv, d, 16, dtype, fill=float("nan"))
+    perm = rng.permutation(pool).tolist()
+    lens_k = [a + b for a, b in seqs]
+    lens_q = [b for _, b in seqs]
+    width = max((l + 15) // 16 for l in lens_k)
+    tables = np.zeros((len(seqs), width), dtype=np.int32)
+    slots_all = []
+    for i, lk in enumerate(lens_k):
+        n = (lk + 15) // 16
+        blocks = [perm.pop() for _ in range(n)]
+        tables[i, :n] = blocks
+        slots = torch.tensor(W.slots_for(blocks, lk), dtype=torch.int64)
+        slots_all.append(slots)
+        k = torch.randn((lk, Hkv, d), generator=g).to(dtype)
+        v = torch.randn((lk, Hkv, d), generator=g).to(dtype)
+        ref.reshape_and_cache(k, v, kc, vc, slots)
+    q = torch.randn((sum(lens_q), Hq, d), generator=g).to(dtype)
+    return dict(q=q, kc=kc, vc=vc, tables=torch.from_numpy(tables), cu_q=W.offsets(lens_q),
+                ctx=torch.tensor(lens_k, dtype=torch.int32), lens_q=lens_q, lens_k=lens_k, slots=slots_all,
+                scale=1.0 / math.sqrt(d))
+
+
+def oracle(c, Hq, Hkv, d):
+    gm = torch.cat(c["slots"]).to(torch.int32)
+    kc, vc = c["kc"].float().nan_to_num(0.0), c["vc"].float().nan_to_num(0.0)   # the oracle reads covered slots only
+    gk = torch.empty((gm.numel(), Hkv, d))
+    gv = torch.empty_like(gk)
+    ref.gather_cached_kv(gk, gv, kc, vc, gm)
+    gk, gv = ref.repeat_kv(gk, Hq // Hkv), ref.repeat_kv(gv, Hq // Hkv)
+    return ref.varlen_attn(c["q"].float(), gk, gv, c["cu_q"], W.offsets(c["lens_k"]), max(c["lens_q"]),
+                           max(c["lens_k"]), c["scale"], True)
+
+
+def run_paged(c, device, lse=False):
+    return K.flash_attn_varlen_paged(c["q"].to(device), c["kc"].to(device), c["vc"].to(device), c["tables"].to(device),
+                                     c["cu_q"].to(device), c["ctx"].to(device), max(c["lens_q"]), max(c["lens_k"]),
+                                     c["scale"], True, return_lse=lse)
+
+
+SEQS = [(0, 5), (0, 64), (100, 33), (1000, 256), (17, 1), (0, 300), (63, 65), (2048, 512), (0, 0), (15, 16)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("heads", [(32, 8, 128), (32, 32, 80), (8, 2, 64), (4, 4, 32), (6, 1, 96)])
+def test_matches_oracle(device, dtype, heads):
+    Hq, Hkv, d = heads
+    c = paged_case(31, SEQS, Hq, Hkv, d, dtype, 420)
+    got = run_paged(c, device).cpu()
+    want = oracle(c, Hq, Hkv, d)
+    assert not torch.isnan(got).any()
+    assert (got.float() - want).abs().max().item() <= TOL[dtype]
+
+
+def test_agrees_with_gather_then_contiguous_prefill_and_lse(device):
+    dtype = torch.bfloat16
+    Hq, Hkv, d = 32, 8, 128
+    c = paged_case(32, [(700, 300), (0, 1024), (3000, 40)], Hq, Hkv, d, dtype, 400)
+    got, lse = run_paged(c, device, lse=True)
+    gm = torch.cat(c["slots"]).to(torch.int32).to(device)
+    gk = torch.empty((gm.numel(), Hkv, d), dtype=dtype, device=device)
+    gv = torch.empty_like(gk)
+    K.gather_cached_kv(gk, gv, c["kc"].to(device), c["vc"].to(device), gm)
+    cu_k = W.offsets(c["lens_k"]).to(device)
+    want, lse2 = K.flash_attn_varlen(c["q"].to(device), gk, gv, c["cu_q"].to(device), cu_k, max(c["lens_q"]),
+                                     max(c["lens_k"]), c["scale"], True, return_lse=True)
+    assert (got.float() - want.float()).abs().max().item() <= TOL[dtype]
+    for i, lq in enumerate(c["lens_q"]):
+        assert torch.allclose(lse[i, :, :lq], lse2[i, :, :lq], atol=2e-3, rtol=1e-4)
+
+
+def test_invariant_under_block_permutation(device):
+    dtype = torch.float16
+    Hq, Hkv, d = 8, 2, 128
+    c = paged_case(33, [(130, 70), (0, 257)], Hq, Hkv, d, dtype, 64)
+    got = run_paged(c, device)
+    perm = torch.randperm(64, generator=torch.Generator().manual_seed(2))
+    kc2, vc2 = torch.empty_like(c["kc"]), torch.empty_like(c["vc"])
+    kc2[perm] = c["kc"]
+    vc2[perm] = c["vc"]
+    nblk = [(l + 15) // 16 for l in c["lens_k"]]
+    t2 = c["tables"].clone()
+    for i, n in enumerate(nblk):
+        t2[i, :n] = perm[c["tables"][i, :n].long()].to(torch.int32)
+    c2 = dict(c, kc=kc2, vc=vc2, tables=t2)
+    assert torch.equal(run_paged(c2, device), got)
+
+
+def test_argument_errors(device):
+    c = paged_case(34, [(0, 20)], 4, 4, 64, torch.float16, 8)
+    with pytest.raises(HipAttnError, match="block-table columns"):
+        K.flash_attn_varlen_paged(c["q"].to(device), c["kc"].to(device), c["vc"].to(device), c["tables"].to(device),
+                                  c["cu_q"].to(device), c["ctx"].to(device), 20, 16 * c["tables"].size(1) + 1,
+                                  c["scale"], True)
+    big = paged_case(35, [(0, 4)], 2, 2, 256, torch.float16, 4)
+    with pytest.raises(HipAttnError, match="head size"):
+        run_paged(big, device)

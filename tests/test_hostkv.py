@@ -203,3 +203,28 @@ def test_cache_geometry():
     import torch
     assert paged.cache_x(torch.float16) == 8 and paged.cache_x(torch.bfloat16) == 8 and paged.cache_x(torch.float32) == 4
     assert paged.cache_block_bytes(16, 8, 128, 32, torch.bfloat16) == ref.cache_block_bytes(16, 8, 128, 32, 2) == 2 * 16 * 8 * 128 * 2 * 32
+
+
+def test_multi_entry_block_tables_extension():
+    """The builder also hands out block tables for multi-token entries when their slots walk the blocks in
+    order (blocks.rs:122-127 slots always do); hand-made slots that do not are flagged."""
+    a = paged.BlockAllocator(16, 32)
+    b = paged.BatchInfoBuilder(16, 4096, 1)
+    a.alloc_seq(1, 40)
+    a.alloc_seq(2, 7)
+    a.alloc_seq(3, 20)
+    b.sched_out(a, 2, list(range(7)), 6)          # single token -> paged rows
+    b.sched_out(a, 1, list(range(40)), 10)        # 30 new tokens
+    b.sched_out(a, 3, list(range(20)), 0)         # prompt
+    bi = b.finish()
+    assert bi.seq_ids == [1, 3, 2] and bi.seqlen_multi == 2
+    assert bi.multi_context_lens.tolist() == [40, 20]
+    assert bi.multi_block_tables.tolist() == [[0, 1, 2], [4, 5, 0]]       # seq 2 took block 3
+    # every gathered slot is reproduced by the table
+    gm = bi.gather_mapping.tolist()
+    want = [bi.multi_block_tables[0, p // 16].item() * 16 + p % 16 for p in range(40)] + \
+           [bi.multi_block_tables[1, p // 16].item() * 16 + p % 16 for p in range(20)]
+    assert gm == want
+    b2 = paged.BatchInfoBuilder(16, 4096, 1)
+    b2.add_entry(9, [0, 1, 2], [5, 6, 7], [32, 34, 33])                    # slots out of order
+    assert b2.finish().multi_block_tables is None
