@@ -131,6 +131,56 @@ def streaming_leg(dev, stream, steps: int) -> dict:
     return res
 
 
+def mixed_step_leg(dev, stream, steps: int) -> dict:
+    """One layer's attention for a mixed continuous-batching step in the Phi-2 shape (32 MHA heads, d 80,
+    fp16): four 512-token chunks with 0/1k/2k/3k tokens already cached plus 120 single-token rows with
+    contexts U[1k,8k] (seed 4) -- `llm::varlen_attn` as one C-ABI call, by the reference's route (scatter,
+    gather, varlen prefill, paged decode) and with the multi-token rows reading the cache through block tables."""
+    import math
+
+    import numpy as np
+    import torch
+
+    from aici_amd import attn, paged
+
+    rng = np.random.default_rng(4)
+    H, d, dt = 32, 80, torch.float16
+    priors, chunk = [0, 1024, 2048, 3072], 512
+    dec = rng.integers(1024, 8193, size=120).tolist()
+    pool = sum((p + chunk + 15) // 16 for p in priors) + sum((c + 15) // 16 for c in dec) + 8
+    alloc = paged.BlockAllocator(16, pool)
+    b = paged.BatchInfoBuilder(16, 1 << 20, 1)
+    sid = 1
+    for p in priors:
+        alloc.alloc_seq(sid, p + chunk)
+        b.sched_out(alloc, sid, rng.integers(0, 1000, size=p + chunk).astype(np.int32), p)
+        sid += 1
+    for c in dec:
+        alloc.alloc_seq(sid, c)
+        b.sched_out(alloc, sid, rng.integers(0, 1000, size=c).astype(np.int32), c - 1)
+        sid += 1
+    bi = b.finish().to(dev)
+    T = bi.tokens.numel()
+    g = torch.Generator(device=dev).manual_seed(4)
+    kc, vc = paged.alloc_gpu_cache_layer(pool, H, d, 16, dt, dev)
+    kc.normal_(generator=g)
+    vc.normal_(generator=g)
+    q, k, v = (torch.randn((T, H, d), generator=g, device=dev, dtype=dt) for _ in range(3))
+    flops = 4 * d * H * sum(chunk * p + chunk * (chunk + 1) // 2 for p in priors)
+    kv_bytes = int(sum(dec)) * 2 * H * d * 2
+    out = {"config": {"workload": "mixed step: 4 x 512 new tokens after 0/1k/2k/3k cached + 120 decode rows ctx "
+                                  "U[1k,8k] (seed 4), 32 MHA heads, d 80, fp16", "tokens": T,
+                      "prefill_flops": flops, "decode_kv_bytes": kv_bytes}}
+    for name, paged_prefill in (("reference_route", False), ("paged_prefill_route", True)):
+        fn = lambda: attn.varlen_attn(q, k, v, bi, kc, vc, 1.0 / math.sqrt(d), paged_prefill=paged_prefill)
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        ms = event_times_ms(fn, steps, stream)
+        out[name] = {"us_per_step": round(sum(ms) / len(ms) * 1e3, 1)}
+    return out
+
+
 def llama_step_leg(dev, stream, steps: int, layers: int, share_cache: bool) -> dict:
     """One full engine step of a Llama-3-8B-shaped model (random weights): 128 sequences decoding
     one token each over contexts U[1024,16384] (seed 5), every layer with its own paged KV cache,
@@ -206,6 +256,8 @@ def main() -> None:
     ap.add_argument("--streaming", action="store_true",
                     help="also time the HBM-bound helper kernels (cache scatter/gather, rotary, norms, "
                          "activation, bias + arg-max) against the HBM roofline")
+    ap.add_argument("--mixed-step", action="store_true",
+                    help="also time one layer's attention for a mixed prefill-chunk + decode step (Phi-2 shape)")
     ap.add_argument("--llama-step", action="store_true",
                     help="also time a full Llama-3-8B-shaped decode step with the AICI mask + greedy stage "
                          "(allocates about 170 GB of HBM)")
@@ -328,6 +380,9 @@ def main() -> None:
     # ---- optional: the streaming helpers -------------------------------------------------------------
     if args.streaming:
         line["streaming"] = streaming_leg(dev, stream, max(20, min(args.steps, 100)))
+
+    if args.mixed_step:
+        line["mixed_step"] = mixed_step_leg(dev, stream, max(20, min(args.steps, 100)))
 
     # ---- optional: the full engine step the decode kernel sits in ---------------------------------
     if args.llama_step:
