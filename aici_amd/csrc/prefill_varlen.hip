@@ -783,11 +783,13 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   };
 
   // P(j).V(j) with the staging for later tiles in its shadow.
-  constexpr int PV_STEPS = NDT * 4;  // step n = (dt, kt, half)
+  constexpr int PV_STEPS = NDT * 4;
   auto pv_stage = [&](bool live, int j, vec8(&pk)[2][2]) {
     const T *vs_base = smem + (j % 3) * TL::STAGE_ELEMS + TL::K_ELEMS;
+    // Step n = (contraction step n / NDT, output tile n % NDT): consecutive MFMAs go to different
+    // accumulators, so none waits for the result of the one before it.
     auto rd = [&](int n) -> vec8 {
-      const int dt = n / 4, kt = (n / 2) % 2, half = n % 2;
+      const int dt = n % NDT, ks = n / NDT, kt = ks / 2, half = ks % 2;
       return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + dt * 32 * TL::VTSTR + kt * 32 + half * 16);
     };
     if (live) {
@@ -798,7 +800,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       for (int n = 0; n < PV_STEPS; n++) {
         if (n + 3 < PV_STEPS) va[(n + 3) % 4] = rd(n + 3);
         __builtin_amdgcn_sched_barrier(0);
-        acc[n / 4] = Mfma32<T>::run(va[n % 4], pk[(n / 2) % 2][n % 2], acc[n / 4]);
+        acc[n % NDT] = Mfma32<T>::run(va[n % 4], pk[(n / NDT) / 2][(n / NDT) % 2], acc[n % NDT]);
         __builtin_amdgcn_sched_barrier(0);
         if (n == 1) {
           if (j + 2 < n_tiles) store_tile((j + 2) % 3);
