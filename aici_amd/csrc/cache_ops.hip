@@ -21,6 +21,27 @@ struct CacheGeom {
   int64_t v_block_stride, v_head_stride;
 };
 
+// One 16-byte run of K and the same elements of V of one token: K's run is adjacent in the cache, V's
+// elements are block_size apart.  SCATTER: token -> cache, else cache -> token.
+template <typename E, bool SCATTER>
+__device__ __forceinline__ void move_token_chunk(E *kp, E *vp, E *kc, E *vc, int block_size) {
+  constexpr int X = 16 / sizeof(E);
+  if (SCATTER) {
+    *reinterpret_cast<uint4 *>(kc) = *reinterpret_cast<const uint4 *>(kp);
+    uint4 vv = *reinterpret_cast<const uint4 *>(vp);
+    const E *ve = reinterpret_cast<const E *>(&vv);
+#pragma unroll
+    for (int j = 0; j < X; j++) vc[(int64_t)j * block_size] = ve[j];
+  } else {
+    *reinterpret_cast<uint4 *>(kp) = *reinterpret_cast<const uint4 *>(kc);
+    uint4 vv;
+    E *ve = reinterpret_cast<E *>(&vv);
+#pragma unroll
+    for (int j = 0; j < X; j++) ve[j] = vc[(int64_t)j * block_size];
+    *reinterpret_cast<uint4 *>(vp) = vv;
+  }
+}
+
 // One 16-byte run of the key cache is `x` consecutive head elements of one
 // token; a thread moves one run of K and the same `x` elements of V.  V's
 // elements of one token are BS apart in the cache.
@@ -48,20 +69,7 @@ __global__ __launch_bounds__(256) void cache_move_vec_kernel(
             ((int64_t)c * g.block_size + off) * X;
     E *vc = value_cache + blk * g.v_block_stride + h * g.v_head_stride +
             (int64_t)c * X * g.block_size + off;
-    if (SCATTER) {
-      *reinterpret_cast<uint4 *>(kc) = *reinterpret_cast<const uint4 *>(kp);
-      uint4 vv = *reinterpret_cast<const uint4 *>(vp);
-      const E *ve = reinterpret_cast<const E *>(&vv);
-#pragma unroll
-      for (int j = 0; j < X; j++) vc[(int64_t)j * g.block_size] = ve[j];
-    } else {
-      *reinterpret_cast<uint4 *>(kp) = *reinterpret_cast<const uint4 *>(kc);
-      uint4 vv;
-      E *ve = reinterpret_cast<E *>(&vv);
-#pragma unroll
-      for (int j = 0; j < X; j++) ve[j] = vc[(int64_t)j * g.block_size];
-      *reinterpret_cast<uint4 *>(vp) = vv;
-    }
+    move_token_chunk<E, SCATTER>(kp, vp, kc, vc, g.block_size);
   }
 }
 
@@ -168,19 +176,107 @@ __global__ __launch_bounds__(256) void cache_move_run8_kernel(
       E *vp = value + token * val_tok_stride + h * val_head_stride + c * X;
       E *kc = key_cache + blk * g.k_block_stride + h * g.k_head_stride + ((int64_t)c * g.block_size + off) * X;
       E *vc = value_cache + blk * g.v_block_stride + h * g.v_head_stride + (int64_t)c * X * g.block_size + off;
+      move_token_chunk<E, SCATTER>(kp, vp, kc, vc, g.block_size);
+    }
+  }
+}
+
+// Coalesced on both sides (2-byte elements, head size a multiple of 64).  The input is token-major,
+// the cache chunk-major, so some side of a direct copy always touches 16-byte pieces 256 bytes apart.
+// Here a wavefront moves one (8 tokens) x (8 chunks = 64 head elements) tile of one head through a
+// private LDS slab: it reads the source in the source's order (128-byte runs), transposes in LDS, and
+// writes the destination in the destination's order -- K as 128-byte runs [chunk][8 tokens], V as the 8
+// tokens (16 bytes) of each of the tile's 64 head elements.  16 tokens per workgroup as in the kernel
+// above; groups that are not a run of 8 slots take its per-token path.
+template <typename Slot, bool SCATTER>
+__global__ __launch_bounds__(256) void cache_move_tile_kernel(
+    uint16_t *__restrict__ key, uint16_t *__restrict__ value, uint16_t *__restrict__ key_cache,
+    uint16_t *__restrict__ value_cache, const Slot *__restrict__ slot_mapping, int64_t num_tokens,
+    int64_t key_tok_stride, int64_t key_head_stride, int64_t val_tok_stride,
+    int64_t val_head_stride, CacheGeom g) {
+  typedef uint16_t E;
+  constexpr int X = 8;
+  constexpr int KP = 72;  // K slab row pitch in elements: 8 chunks + 16 bytes, keeps the transposed 16-byte reads apart
+  constexpr int VP = 64;  // V slab row pitch: the 2-byte column accesses of a wavefront fall in one row
+  __shared__ __attribute__((aligned(16))) E slab[4][8 * KP + 8 * VP];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  E *ks = slab[wave], *vs = slab[wave] + 8 * KP;
+  const int64_t wg_t0 = (int64_t)blockIdx.x * 16;
+  const int chunks_per_head = g.head_size / X;
+  const int groups_per_head = chunks_per_head / 8;
+  const int items_per_half = g.num_heads * groups_per_head;
+  int64_t run_slot[2];
+#pragma unroll
+  for (int half = 0; half < 2; half++) {
+    const int64_t t0 = wg_t0 + 8 * half;
+    run_slot[half] = -1;
+    if (t0 + 8 <= num_tokens) {
+      const int64_t slot0 = (int64_t)slot_mapping[t0];
+      bool run = slot0 >= 0 && slot0 % 8 == 0 && slot0 / g.block_size < g.num_blocks;
+      if (run) {
+#pragma unroll
+        for (int i = 1; i < 8; i++) run = run && (int64_t)slot_mapping[t0 + i] == slot0 + i;
+      }
+      if (run) run_slot[half] = slot0;
+    }
+  }
+  const int hi = lane >> 3, lo = lane & 7;
+  for (int item = wave; item < 2 * items_per_half; item += 4) {  // uniform per wavefront
+    const int half = item / items_per_half;
+    const int rem = item % items_per_half;
+    const int h = rem / groups_per_head, cg = rem % groups_per_head;
+    const int64_t t0 = wg_t0 + 8 * half;
+    const int64_t slot0 = half == 0 ? run_slot[0] : run_slot[1];
+    if (slot0 >= 0) {
+      const int64_t blk = slot0 / g.block_size;
+      const int off0 = (int)(slot0 % g.block_size);
+      E *kc_base = key_cache + blk * g.k_block_stride + h * g.k_head_stride;
+      E *vc_base = value_cache + blk * g.v_block_stride + h * g.v_head_stride;
+      // token-major side: lane (token hi, chunk lo); cache side: lane (chunk hi, token lo) for K,
+      // lane (chunk hi, element lo) for V
+      E *k_tok = key + (t0 + hi) * key_tok_stride + h * key_head_stride + (cg * 8 + lo) * X;
+      E *v_tok = value + (t0 + hi) * val_tok_stride + h * val_head_stride + (cg * 8 + lo) * X;
+      E *k_cache = kc_base + ((int64_t)(cg * 8 + hi) * g.block_size + off0 + lo) * X;
+      E *v_cache = vc_base + (int64_t)((cg * 8 + hi) * X + lo) * g.block_size + off0;
       if (SCATTER) {
-        *reinterpret_cast<uint4 *>(kc) = *reinterpret_cast<const uint4 *>(kp);
-        uint4 vv = *reinterpret_cast<const uint4 *>(vp);
-        const E *ve = reinterpret_cast<const E *>(&vv);
+        *reinterpret_cast<uint4 *>(ks + hi * KP + lo * X) = *reinterpret_cast<const uint4 *>(k_tok);
+        *reinterpret_cast<uint4 *>(vs + hi * VP + lo * X) = *reinterpret_cast<const uint4 *>(v_tok);
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the slab is private to this wavefront
+        *reinterpret_cast<uint4 *>(k_cache) = *reinterpret_cast<const uint4 *>(ks + lo * KP + hi * X);
+        uint4 o;
+        E *oe = reinterpret_cast<E *>(&o);
 #pragma unroll
-        for (int j = 0; j < X; j++) vc[(int64_t)j * g.block_size] = ve[j];
+        for (int t = 0; t < 8; t++) oe[t] = vs[t * VP + lane];  // element (hi, lo) of token t
+        *reinterpret_cast<uint4 *>(v_cache) = o;
       } else {
-        *reinterpret_cast<uint4 *>(kp) = *reinterpret_cast<const uint4 *>(kc);
-        uint4 vv;
-        E *ve = reinterpret_cast<E *>(&vv);
+        *reinterpret_cast<uint4 *>(ks + lo * KP + hi * X) = *reinterpret_cast<const uint4 *>(k_cache);
+        const uint4 vin = *reinterpret_cast<const uint4 *>(v_cache);
+        const E *ve = reinterpret_cast<const E *>(&vin);
 #pragma unroll
-        for (int j = 0; j < X; j++) ve[j] = vc[(int64_t)j * g.block_size];
-        *reinterpret_cast<uint4 *>(vp) = vv;
+        for (int t = 0; t < 8; t++) vs[t * VP + lane] = ve[t];
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        *reinterpret_cast<uint4 *>(k_tok) = *reinterpret_cast<const uint4 *>(ks + hi * KP + lo * X);
+        *reinterpret_cast<uint4 *>(v_tok) = *reinterpret_cast<const uint4 *>(vs + hi * VP + lo * X);
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // slab reads done before the next item overwrites it
+      continue;
+    }
+    // per-token path for this group of 8: lane = chunk of the 64-element group, tokens in turn
+    for (int t = 0; t < 8; t++) {
+      const int64_t token = t0 + t;
+      if (token >= num_tokens) break;
+      const int64_t slot = (int64_t)slot_mapping[token];
+      if (slot < 0) continue;
+      const int64_t blk = slot / g.block_size;
+      if (blk >= g.num_blocks) continue;
+      const int off = (int)(slot % g.block_size);
+      if (lane < 8) {
+        const int c = cg * 8 + lane;
+        E *kp = key + token * key_tok_stride + h * key_head_stride + c * X;
+        E *vp = value + token * val_tok_stride + h * val_head_stride + c * X;
+        E *kc = key_cache + blk * g.k_block_stride + h * g.k_head_stride + ((int64_t)c * g.block_size + off) * X;
+        E *vc = value_cache + blk * g.v_block_stride + h * g.v_head_stride + (int64_t)c * X * g.block_size + off;
+        move_token_chunk<E, SCATTER>(kp, vp, kc, vc, g.block_size);
       }
     }
   }
@@ -272,6 +368,14 @@ void launch_move(const hipattn_tensor *key, const hipattn_tensor *value,
     // long inputs (prompts): 8-token workgroups with the transposing fast path
     if (vec && T >= 1024 && g.block_size % 8 == 0 && aligned16(vc) && g.v_block_stride % 8 == 0 &&
         g.v_head_stride % 8 == 0) {
+      // The LDS-transposing kernel pays off for the scatter (its stores become whole lines) once there are
+      // enough 16-token workgroups to hide its load -> LDS -> store chains; the gather is as fast without it.
+      if (SCATTER && g.head_size % 64 == 0 && T >= 16384 && getenv("HIPATTN_CACHE_MOVE_NO_LDS") == nullptr) {
+        cache_move_tile_kernel<Slot, SCATTER><<<dim3((unsigned)((T + 15) / 16)), 256, 0, stream>>>(
+            kp, vp, kc, vc, sp, T, key->strides[0], key->strides[1], value->strides[0], value->strides[1], g);
+        check_launch(SCATTER ? "reshape_and_cache" : "gather_cached_kv");
+        return;
+      }
       int n = g.num_heads * (g.head_size / X);
       int threads = n < 256 ? ((n + 63) / 64) * 64 : 256;
       cache_move_run8_kernel<Slot, SCATTER><<<dim3((unsigned)((T + 15) / 16)), threads, 0, stream>>>(
