@@ -902,13 +902,14 @@ void launch_prefill(PrefillParams p, hipStream_t stream) {
 
 template <typename T, int HDP>
 void pick_qt(const PrefillParams &p, int64_t total_q, hipStream_t stream) {
-  // 256-row workgroups halve LDS traffic per flop but need enough rows to
-  // fill the 256 CUs; small launches use 128-row workgroups.
+  // The eight-wavefront kernel (256-row workgroups) wins from a few hundred workgroups up -- measured
+  // 4 x 512 tokens x 32 heads: 28 vs 33 us, 2 x 2048: 90 vs 144 us; only the smallest launches (4 sequences
+  // of 128..512 tokens: 24.6 vs 22.7 us) prefer 128-row workgroups.
   if constexpr (HDP <= 128) {
     const int64_t wg256 = (total_q / 256 + p.batch) * p.Hq;
     const char *force = getenv("HIPATTN_PREFILL_KERNEL");  // tuning aid: "w8", "qt2" or "qt1"
     // the eight-wavefront kernel addresses a tile's 64 rows with 32-bit byte offsets
-    const bool big = wg256 >= 2 * 256 && p.k_row < (1 << 23) && p.v_row < (1 << 23);
+    const bool big = wg256 >= 320 && p.k_row < (1 << 23) && p.v_row < (1 << 23);
     if ((force ? !strcmp(force, "w8") : big) && p.k_row < (1 << 23) && p.v_row < (1 << 23)) {
       launch_prefill_w8<T, HDP>(p, stream);
       return;
