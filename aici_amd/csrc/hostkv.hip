@@ -56,6 +56,13 @@ struct hipattn_batch_builder {
     std::vector<int64_t> q_pos;
     std::vector<int32_t> q_tok;
     std::vector<int64_t> kv_slots;
+    // Single-token entries added through add_seq keep only the sequence's block list: building the slot
+    // of every context position (O(context) per sequence and step) is not needed for rows that go to the
+    // paged kernel, which reads block tables.
+    bool by_blocks = false;
+    std::vector<int64_t> blocks;
+    int64_t k_len = 0;
+    int64_t num_keys() const { return by_blocks ? k_len : (int64_t)kv_slots.size(); }
   };
   int64_t block_size, max_model_len;
   int paged_v;
@@ -270,12 +277,22 @@ extern "C" char *hipattn_batch_builder_add_seq(hipattn_batch_builder *b, const h
       e.q_pos.push_back(i);
       e.q_tok.push_back(seq_tokens[i]);
     }
-    e.kv_slots.resize((size_t)seq_len);
-    char *err = hipattn_block_allocator_get_block_idxes(a, seq_id, seq_len, e.kv_slots.data());
-    if (err) {
-      std::string msg(err);
-      free(err);
-      fail("%s", msg.c_str());
+    if (b->paged_v > 0 && q_len == 1) {
+      auto it = a->seq_blocks.find(seq_id);
+      const int64_t need = a->num_blocks_for(seq_len);
+      HA_CHECK(it != a->seq_blocks.end() && (int64_t)it->second.size() >= need,
+               "sequence %lld holds fewer blocks than %lld tokens need", (long long)seq_id, (long long)seq_len);
+      e.by_blocks = true;
+      e.blocks.assign(it->second.begin(), it->second.begin() + need);
+      e.k_len = seq_len;
+    } else {
+      e.kv_slots.resize((size_t)seq_len);
+      char *err = hipattn_block_allocator_get_block_idxes(a, seq_id, seq_len, e.kv_slots.data());
+      if (err) {
+        std::string msg(err);
+        free(err);
+        fail("%s", msg.c_str());
+      }
     }
     b->entries.push_back(std::move(e));
   });
@@ -305,13 +322,16 @@ extern "C" char *hipattn_batch_builder_finish(hipattn_batch_builder *b, hipattn_
     for (size_t idx = 0; idx < b->entries.size(); idx++) {
       const Entry &e = b->entries[idx];
       b->seq_ids.push_back(e.seq_id);
-      const size_t off = e.kv_slots.size() - e.q_tok.size();
+      const size_t off = (size_t)e.num_keys() - e.q_tok.size();
       for (size_t qi = 0; qi < e.q_tok.size(); qi++) {
         HA_CHECK(e.q_pos[qi] < b->max_model_len, "position %lld is past max_model_len %lld", (long long)e.q_pos[qi],
                  (long long)b->max_model_len);
         b->positions.push_back(e.q_pos[qi]);
         b->tokens.push_back(e.q_tok[qi]);
-        b->slot_mapping.push_back((int32_t)e.kv_slots[off + qi]);
+        const int64_t pos = (int64_t)(off + qi);
+        const int64_t slot = e.by_blocks ? e.blocks[(size_t)(pos / b->block_size)] * b->block_size + pos % b->block_size
+                                         : e.kv_slots[off + qi];
+        b->slot_mapping.push_back((int32_t)slot);
       }
       b->logit_idxs.push_back((int32_t)b->tokens.size() - 1);
       if (idx < num_multi) {
@@ -333,8 +353,10 @@ extern "C" char *hipattn_batch_builder_finish(hipattn_batch_builder *b, hipattn_
         multi_tables.push_back(std::move(row));
         b->multi_ctx_lens.push_back((int32_t)e.kv_slots.size());
       } else {
-        b->ctx_lens.push_back((int32_t)e.kv_slots.size());
+        b->ctx_lens.push_back((int32_t)e.num_keys());
         std::vector<int32_t> row;
+        if (e.by_blocks)
+          for (int64_t blk : e.blocks) row.push_back((int32_t)blk);
         for (size_t i = 0; i < e.kv_slots.size(); i += (size_t)b->block_size) {
           const int64_t slot = e.kv_slots[i];
           HA_CHECK(slot % b->block_size == 0, "slot %lld at a block boundary is not block-aligned", (long long)slot);

@@ -29,7 +29,7 @@ class BlockAllocator:
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
-        if h:
+        if h and _lib is not None:  # module globals are gone at interpreter shutdown
             _lib.load().hipattn_block_allocator_free(h)
 
     def get_num_free_blocks(self) -> int:
@@ -127,7 +127,7 @@ class BatchInfoBuilder:
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
-        if h:
+        if h and _lib is not None:
             _lib.load().hipattn_batch_builder_free(h)
 
     def add_entry(self, seq_id: int, query_positions: Sequence[int], query_tokens: Sequence[int],
