@@ -68,6 +68,36 @@ def cpu_baseline_decode(c_cpu, rows, threads: int) -> dict:
                       "bytes counted as for the GPU (bf16 K/V once per kv head)"}
 
 
+def memory_system_leg(dev, stream, steps: int) -> dict:
+    """What this device's memory system delivers to the simplest possible kernels (16 bytes per lane,
+    grid-stride), beside the published 8 TB/s: a 1 GiB read, a 1 GiB copy, a 1 GiB fill, and the read of
+    a 1.3 GB buffer in shuffled 4 KiB chunks -- the granule and footprint of the decode leg's K/V blocks."""
+    import torch
+    from aici_amd import kernels as K
+
+    n = 1 << 30
+    src = torch.empty((n,), dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    big = torch.empty((20000 * 16 * 4096,), dtype=torch.uint8, device=dev).fill_(1)  # 20k blocks x 8 heads x (K, V)
+    g = torch.Generator().manual_seed(17)
+    order = torch.randperm(big.numel() // 4096, generator=g)[:154_000].to(torch.int32).to(dev)  # ~631 MB of distinct chunks
+    out = {}
+
+    def run(name, fn, nbytes):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        ts = event_times_ms(fn, steps, stream)
+        ms = sum(ts) / len(ts)
+        out[name] = {"GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1), "us": round(ms * 1e3, 1), "bytes": nbytes}
+
+    run("read_1GiB", lambda: K.stream_probe("read", None, src), n)
+    run("copy_1GiB_read_plus_write", lambda: K.stream_probe("copy", dst, src), 2 * n)
+    run("fill_1GiB", lambda: K.stream_probe("fill", dst, None), n)
+    run("read_4KiB_chunks_shuffled", lambda: K.stream_probe("read_chunks", None, big, order), order.numel() * 4096)
+    return out
+
+
 def streaming_leg(dev, stream, steps: int) -> dict:
     """The HBM-bound helpers of the path at the sizes of the prefill (config 3: 32768 tokens) and of the
     full decode step (config 5: 128 x 128256 logits): algorithmic bytes / average launch time (HIP events)."""
@@ -263,6 +293,9 @@ def main() -> None:
                          "(allocates about 170 GB of HBM)")
     ap.add_argument("--llama-layers", type=int, default=32)
     ap.add_argument("--llama-share-cache", action="store_true", help="all layers read one layer's KV cache")
+    ap.add_argument("--memory-system", action="store_true",
+                    help="also time plain read / copy / fill kernels and a shuffled 4 KiB-chunk read: the "
+                         "attainable rates beside the 8 TB/s peak")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (torch copy_) so that FETCH_SIZE / WRITE_SIZE "
                          "read under rocprofv3 --pmc can be scaled against a kernel of known traffic")
@@ -380,6 +413,9 @@ def main() -> None:
     # ---- optional: the streaming helpers -------------------------------------------------------------
     if args.streaming:
         line["streaming"] = streaming_leg(dev, stream, max(20, min(args.steps, 100)))
+
+    if args.memory_system:
+        line["memory_system"] = memory_system_leg(dev, stream, 20)
 
     if args.mixed_step:
         line["mixed_step"] = mixed_step_leg(dev, stream, max(20, min(args.steps, 100)))
