@@ -15,6 +15,18 @@ from tests.common import TOL, kat_inputs, load_kat, round4
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["auto", "eight_wavefronts", "four_wavefronts"])
+def kernel_choice(request, monkeypatch):
+    """The forward pass has two kernels (256-row workgroups of eight wavefronts for head sizes up to
+    128, 128-row workgroups of four) and picks by launch size; every test runs under the library's
+    own choice and with each one forced (head sizes above 128 always take the second)."""
+    if request.param == "auto":
+        monkeypatch.delenv("HIPATTN_PREFILL_KERNEL", raising=False)
+    else:
+        monkeypatch.setenv("HIPATTN_PREFILL_KERNEL", "w8" if request.param == "eight_wavefronts" else "qt1")
+    return request.param
+
+
 def run(p: W.PrefillInputs, device, causal=True, **kw):
     d = p.to(device)
     return K.flash_attn_varlen(d.q, d.k, d.v, d.cu_q, d.cu_k, p.max_q, p.max_k, p.scale, causal, **kw)
