@@ -81,7 +81,11 @@ struct PrefillParams {
   int lse_pitch;  // elements between (batch, head) rows of lse
   int n_qblocks;
   float scale_log2;
-  int causal;
+  int causal;  // win_left < 0 && win_right == 0
+  // Query row i (0-based in its sequence) sees key j iff i + off - win_left <= j <= i + off + win_right,
+  // off = Lk - Lq; a negative bound is no bound (flash_attn/softmax.h:142-179, flash_api.cpp:113-120).
+  // Only prefill_varlen_kernel reads these; the eight-wavefront kernel takes causal or unmasked launches.
+  int win_left, win_right;
   // K/V read straight from the paged cache (prefill_varlen_w8_kernel<..., PAGED = true>): k and v are
   // the caches, position p of sequence b lives in block block_tables[b][p / 16] at offset p % 16.
   const int32_t *block_tables;
@@ -184,11 +188,14 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
   if (p.seqused_k) Lk = min(Lk, p.seqused_k[b]);
   const int wg_row0 = qb * BM;
   if (wg_row0 >= Lq) return;
-  const int off = Lk - Lq;  // bottom-right alignment of the causal mask
+  const int off = Lk - Lq;  // bottom-right alignment of the mask
   const int wg_last_row = min(wg_row0 + BM, Lq) - 1;
-  int kmax = p.causal ? min(Lk, wg_last_row + off + 1) : Lk;
+  const bool bound_hi = p.win_right >= 0, bound_lo = p.win_left >= 0;
+  int kmax = bound_hi ? min((int64_t)Lk, (int64_t)wg_last_row + off + p.win_right + 1) : Lk;
   if (kmax < 0) kmax = 0;
   const int n_tiles = (kmax + BN - 1) / BN;
+  // first tile that any row of the workgroup can see
+  const int first_tile = bound_lo ? (int)max((int64_t)0, ((int64_t)wg_row0 + off - p.win_left)) / BN : 0;
 
   const int wave_row0 = wg_row0 + wave * (QT * 32);
   const int wave_last_row = wave_row0 + QT * 32 - 1;
@@ -255,10 +262,10 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
     }
   };
 
-  if (n_tiles > 0) {
-    load_tile(0);
-    store_tile(0);
-    if (n_tiles > 1) load_tile(1);
+  if (n_tiles > first_tile) {
+    load_tile(first_tile);
+    store_tile(first_tile & 1);
+    if (n_tiles > first_tile + 1) load_tile(first_tile + 1);
   }
   __syncthreads();
 
@@ -267,19 +274,21 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
   const int rh = (lane >> 4) & 1, li = lane & 15;
   const int v_lane_off = (4 * g + (li >> 2)) * TL::VSTR + 16 * rh + 4 * (li & 3);
 
-  for (int j = 0; j < n_tiles; j++) {
+  for (int j = first_tile; j < n_tiles; j++) {
     const int cur = j & 1;
     if (j + 1 < n_tiles) store_tile(cur ^ 1);
     if (j + 2 < n_tiles) load_tile(j + 2);
 
     const int k0 = j * BN;
-    // Wave-level view of this tile: skip it if it lies entirely past the
-    // diagonal of every row this wave owns.
-    const bool skip = (wave_row0 >= Lq) || (p.causal && k0 > wave_last_row + off);
+    // Wave-level view of this tile: skip it if it lies entirely outside the
+    // window of every row this wave owns.
+    const bool skip = (wave_row0 >= Lq) || (bound_hi && k0 > (int64_t)wave_last_row + off + p.win_right) ||
+                      (bound_lo && k0 + BN - 1 < (int64_t)wave_row0 + off - p.win_left);
     if (!skip) {
       const T *ks_base = smem + cur * TL::STAGE_ELEMS;
       const T *vs_base = ks_base + TL::K_ELEMS;
-      const bool need_mask = (k0 + BN > Lk) || (p.causal && k0 + BN - 1 > wave_row0 + off);
+      const bool need_mask = (k0 + BN > Lk) || (bound_hi && k0 + BN - 1 > (int64_t)wave_row0 + off + p.win_right) ||
+                             (bound_lo && k0 < (int64_t)wave_last_row + off - p.win_left);
 
       // S^T = K . Q^T for the 32 keys of half-tile hf: rows = keys, one query per lane column.
       auto qk = [&](int hf, f32x16_t(&s)[QT]) {
@@ -300,12 +309,12 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
         for (int qt = 0; qt < QT; qt++) {
           if (need_mask) {
             const int row = wave_row0 + qt * 32 + c;
-            int limit = p.causal ? row + off : Lk - 1;
-            limit = min(limit, Lk - 1);
+            const int limit = bound_hi ? (int)min((int64_t)Lk - 1, (int64_t)row + off + p.win_right) : Lk - 1;
+            const int first = bound_lo ? (int)max((int64_t)0, (int64_t)row + off - p.win_left) : 0;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
               const int key = k0 + hf * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
-              if (key > limit) s[qt][i] = -INFINITY;
+              if (key > limit || key < first) s[qt][i] = -INFINITY;
             }
           }
           float mx = s[qt][0];
@@ -915,7 +924,9 @@ void pick_qt(const PrefillParams &p, int64_t total_q, hipStream_t stream) {
     const char *force = getenv("HIPATTN_PREFILL_KERNEL");  // tuning aid: "w8", "qt2" or "qt1"
     // the eight-wavefront kernel addresses a tile's 64 rows with 32-bit byte offsets
     const bool big = wg256 >= 320 && p.k_row < (1 << 23) && p.v_row < (1 << 23);
-    if ((force ? !strcmp(force, "w8") : big) && p.k_row < (1 << 23) && p.v_row < (1 << 23)) {
+    // it knows the causal mask and no mask; other windows go to the four-wavefront kernel
+    const bool plain = p.win_left < 0 && p.win_right <= 0;
+    if (plain && (force ? !strcmp(force, "w8") : big) && p.k_row < (1 << 23) && p.v_row < (1 << 23)) {
       launch_prefill_w8<T, HDP>(p, stream);
       return;
     }
@@ -998,10 +1009,12 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
   }
   HA_CHECK(p_dropout == 0.f, "mha_varlen_fwd: dropout is not supported (inference only)");
   HA_CHECK(scale > 0.f, "mha_varlen_fwd: softmax_scale must be positive");
-  // The reference turns is_causal into window (-1, 0); other windows are local
-  // attention, which rLLM never asks for (lib.rs:93-95).
-  HA_CHECK(win_left < 0 && (win_right < 0 || (win_right == 0)), "mha_varlen_fwd: sliding-window attention is not supported");
-  if (win_right == 0) causal = true;
+  // flash_api.cpp:466, 113-120: causal is the window (-inf, 0]; one given bound leaves the other open.
+  // rLLM itself only ever passes (-1, -1) (lib.rs:96-97).
+  if (causal) win_right = 0;
+  if (win_left < 0) win_left = -1;
+  if (win_right < 0) win_right = -1;
+  causal = win_left < 0 && win_right == 0;
   HA_CHECK(max_q >= 0 && max_k >= 0, "mha_varlen_fwd: negative max_seqlen");
   if (lse) {
     check_tensor(lse, "softmax_lse", 3);
@@ -1052,6 +1065,8 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
   p.lse_pitch = lse ? (int)lse->sizes[2] : 0;
   p.scale_log2 = scale * kLog2e;
   p.causal = causal ? 1 : 0;
+  p.win_left = win_left;
+  p.win_right = win_right;
   if (q->dtype == HIPATTN_F16) dispatch_hd<half_t>(p, total_q, stream);
   else dispatch_hd<bf16_t>(p, total_q, stream);
 }
@@ -1156,6 +1171,8 @@ void mha_varlen_fwd_paged_impl(const hipattn_tensor *q, const hipattn_tensor *ke
   p.lse_pitch = lse ? (int)lse->sizes[2] : 0;
   p.scale_log2 = scale * kLog2e;
   p.causal = causal ? 1 : 0;
+  p.win_left = -1;
+  p.win_right = causal ? 0 : -1;
   p.block_tables = static_cast<const int32_t *>(block_tables->data);
   p.context_lens = static_cast<const int32_t *>(context_lens->data);
   p.table_stride = block_tables->strides[0];

@@ -55,15 +55,18 @@ def _stream(ref: torch.Tensor):
 
 def flash_attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, seqlens_q: torch.Tensor,
                       seqlens_k: torch.Tensor, max_seqlen_q: int, max_seqlen_k: int, softmax_scale: float,
-                      causal: bool, *, return_lse: bool = False, seqused_k: Optional[torch.Tensor] = None):
-    """lib.rs:69-104.  q [total_q, Hq, d], k/v [total_k, Hkv, d]; returns [total_q, Hq, d]."""
+                      causal: bool, *, return_lse: bool = False, seqused_k: Optional[torch.Tensor] = None,
+                      window=(-1, -1)):
+    """lib.rs:69-104.  q [total_q, Hq, d], k/v [total_k, Hkv, d]; returns [total_q, Hq, d].
+    window = (left, right) of mha_varlen_fwd_C (flash_api.cpp:635-636); rLLM always passes (-1, -1)."""
     out = torch.empty((q.size(0), q.size(1), q.size(2)), dtype=q.dtype, device=q.device)
     lse = None
     if return_lse:
         lse = torch.empty((seqlens_q.numel() - 1, q.size(1), max_seqlen_q), dtype=torch.float32, device=q.device)
     call("hipattn_mha_varlen_fwd", _desc(q, "q"), _desc(k, "k"), _desc(v, "v"), _desc(seqlens_q, "seqlens_q"),
          _desc(seqlens_k, "seqlens_k"), _desc(seqused_k, "seqused_k"), int(max_seqlen_q), int(max_seqlen_k), 0.0,
-         float(softmax_scale), False, bool(causal), -1, -1, _desc(out, "out"), _desc(lse, "lse"), _stream(q))
+         float(softmax_scale), False, bool(causal), int(window[0]), int(window[1]), _desc(out, "out"),
+         _desc(lse, "lse"), _stream(q))
     return (out, lse) if return_lse else out
 
 

@@ -73,8 +73,11 @@ const char *hipattn_version(void);
  * out [total_q, Hq, d] caller-allocated, softmax_lse f32 [b, Hq, max_seqlen_q]
  * or NULL.  fp16/bf16, d % 8 == 0, d <= 256, Hq % Hkv == 0.  Causal masking is
  * bottom-right aligned: key j is visible to query i iff j <= i + (Lk - Lq)
- * (flash_attn/softmax.h:159-160).  p_dropout must be 0 and the window must be
- * (-1,-1) or, with is_causal, (-1,0); zero_tensors clears out (and lse) first. */
+ * (flash_attn/softmax.h:159-160).  window_size_left / window_size_right as in
+ * the reference (flash_api.cpp:113-120,466; softmax.h:155-166): with bounds
+ * (l, r) key j is visible iff i + (Lk - Lq) - l <= j <= i + (Lk - Lq) + r, a
+ * negative bound is no bound, is_causal forces r = 0; rLLM passes (-1,-1).
+ * p_dropout must be 0; zero_tensors clears out (and lse) first. */
 char *hipattn_mha_varlen_fwd(const hipattn_tensor *q, const hipattn_tensor *k,
                              const hipattn_tensor *v,
                              const hipattn_tensor *cu_seqlens_q,

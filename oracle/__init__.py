@@ -28,6 +28,12 @@ How each function is pinned (tests/test_oracle_*.py):
                          llama.rs; closed forms (zeroed output projections,
                          one-token sequences) and prefill-then-decode ==
                          one longer prefill (tests/test_oracle_llama.py).
+  sliding window         (varlen_attn_fp64's `window`; the GPU entry point's
+                         window_size_left/right, which rLLM never sets and the
+                         CPU refkernels lack) no reference vector exists: pinned
+                         by its special cases -- open = unmasked, (-1, 0) =
+                         causal, (0, 0) = one key per row, wider than the
+                         sequence = none -- and a scalar triple loop.
 No function is left "parity unpinned" except the last-ulp behaviour of
 libtorch-CPU SDPA, which is irrelevant at the 5e-3 / 2e-2 gates and is
 bracketed by the fp64 brute force.

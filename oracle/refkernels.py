@@ -105,11 +105,28 @@ def varlen_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, seqlens_q: to
     return torch.cat(outs, 0)
 
 
-def varlen_attn_fp64(q, k, v, seqlens_q, seqlens_k, softmax_scale: float, causal: bool = True) -> torch.Tensor:
+def window_bounds(causal: bool, window=(-1, -1)):
+    """flash_api.cpp:466 and 113-120: causal forces the right bound to 0; a negative bound is no
+    bound.  Returns (left, right) with None for "open"."""
+    left, right = window
+    if causal:
+        right = 0
+    return (left if left >= 0 else None), (right if right >= 0 else None)
+
+
+def varlen_attn_fp64(q, k, v, seqlens_q, seqlens_k, softmax_scale: float, causal: bool = True,
+                     window=(-1, -1)) -> torch.Tensor:
     """Independent statement of the same function: explicit fp64 softmax(QK^T*scale + bias)V
     with the visibility rule written out as an index comparison (flash_attn/softmax.h:159-160).
     GQA-aware (kv head = q head // n_rep).  Rows with no visible key give 0, as the GPU
-    kernel does (flash_fwd_kernel.h:629-668)."""
+    kernel does (flash_fwd_kernel.h:629-668).
+
+    window = (left, right): the sliding window of the GPU kernel's C entry point, which rLLM never
+    sets (tch-cuda/src/lib.rs:96-97 passes -1, -1) and the CPU refkernels do not know: row i sees
+    column j iff i + off - left <= j <= i + off + right, off = Lk - Lq (softmax.h:155-166,
+    `col_idx_limit_left/right`).  No vector of the reference pins the window; the tests pin it by
+    its special cases (open window = unmasked, (-1, 0) = causal, (0, 0) = one key per row) and a
+    scalar triple loop."""
     sq, sk = seqlens_q.tolist(), seqlens_k.tolist()
     Hq, Hkv = q.shape[1], k.shape[1]
     n_rep = Hq // Hkv
@@ -123,7 +140,12 @@ def varlen_attn_fp64(q, k, v, seqlens_q, seqlens_k, softmax_scale: float, causal
         vi = v[sk[i]:sk[i] + lk].double()
         rows = torch.arange(lq).reshape(lq, 1)
         cols = torch.arange(lk).reshape(1, lk)
-        visible = (cols <= rows + (lk - lq)) if causal else torch.ones(lq, lk, dtype=torch.bool)
+        left, right = window_bounds(causal, window)
+        visible = torch.ones(lq, lk, dtype=torch.bool)
+        if right is not None:
+            visible &= cols <= rows + (lk - lq) + right
+        if left is not None:
+            visible &= cols >= rows + (lk - lq) - left
         for h in range(Hq):
             s = qi[:, h, :] @ ki[:, h // n_rep, :].T * softmax_scale
             s = s.masked_fill(~visible, float("-inf"))

@@ -211,3 +211,40 @@ def test_paged_attention_invariant_under_block_permutation_and_equals_prefill_la
     qq[-1] = q[s]
     full = ref.varlen_attn(qq, ref.repeat_kv(kk, n_rep), ref.repeat_kv(vv, n_rep), cu([c]), cu([c]), c, c, 0.25, True)
     assert torch.allclose(full[-1], out[s], atol=1e-6)
+
+
+def test_sliding_window_special_cases_and_triple_loop():
+    """The window of mha_varlen_fwd_C (softmax.h:155-166) in the fp64 statement: open = unmasked,
+    (-1, 0) = causal, causal overrides the right bound, (0, 0) = exactly one key per row, a window
+    wider than the sequence = no window, and a scalar triple loop over a chunk with prior context."""
+    g = torch.Generator().manual_seed(31)
+    lq, lk, H, d = 5, 9, 2, 4
+    q = torch.randn((lq, H, d), generator=g)
+    k, v = (torch.randn((lk, H, d), generator=g) for _ in range(2))
+    a = dict(seqlens_q=cu([lq]), seqlens_k=cu([lk]), softmax_scale=0.41)
+    f = lambda causal, window: ref.varlen_attn_fp64(q, k, v, causal=causal, window=window, **a)
+    assert torch.equal(f(False, (-1, -1)), ref.varlen_attn_fp64(q, k, v, causal=False, **a))
+    assert torch.equal(f(False, (-1, 0)), f(True, (-1, -1)))
+    assert torch.equal(f(True, (-1, 3)), f(True, (-1, -1)))
+    assert torch.equal(f(False, (100, 100)), f(False, (-1, -1)))
+    assert torch.equal(f(True, (100, -1)), f(True, (-1, -1)))
+    one = f(False, (0, 0))  # row i sees only key i + (lk - lq)
+    assert torch.allclose(one, v[lk - lq:].double(), atol=1e-12)
+    for causal, (wl, wr) in [(False, (2, 1)), (True, (3, -1)), (False, (-1, 2)), (False, (1, -1)), (False, (0, 3))]:
+        want = torch.zeros(lq, H, d, dtype=torch.float64)
+        for i in range(lq):
+            for h in range(H):
+                ws = []
+                for j in range(lk):
+                    hi_ok = True if (wr < 0 and not causal) else j <= i + (lk - lq) + (0 if causal else wr)
+                    lo_ok = True if wl < 0 else j >= i + (lk - lq) - wl
+                    ws.append(math.exp(0.41 * sum(float(q[i, h, e]) * float(k[j, h, e]) for e in range(d)))
+                              if hi_ok and lo_ok else 0.0)
+                z = sum(ws)
+                for e in range(d):
+                    want[i, h, e] = sum(w * float(v[j, h, e]) for j, w in enumerate(ws)) / z if z > 0 else 0.0
+        assert (f(causal, (wl, wr)) - want).abs().max().item() < 1e-12, (causal, wl, wr)
+    # more queries than keys: rows whose window lies before key 0 give zeros
+    q2 = torch.randn((6, H, d), generator=g)
+    o = ref.varlen_attn_fp64(q2, k[:2], v[:2], cu([6]), cu([2]), 0.41, causal=False, window=(1, 0))
+    assert torch.all(o[:3] == 0) and not torch.all(o[4] == 0)
