@@ -197,3 +197,70 @@ def alloc_gpu_cache_layer(num_blocks: int, num_kv_heads: int, head_size: int, bl
     k = torch.empty((num_blocks, num_kv_heads, head_size // x, block_size, x), dtype=dtype, device=device)
     v = torch.empty((num_blocks, num_kv_heads, head_size, block_size), dtype=dtype, device=device)
     return k, v
+
+
+class CacheEngine:
+    """cache_engine.rs:16-176: the per-layer paged K/V caches on the device, their host-side swap
+    space, the side stream that block swaps run on with one event per layer, and copy-on-write
+    block copies.  Host caches are pinned (allocated so, never registered afterwards)."""
+
+    def __init__(self, num_layers: int, num_kv_heads: int, head_size: int, block_size: int, dtype: torch.dtype,
+                 num_gpu_blocks: int, num_cpu_blocks: int, device):
+        from . import kernels
+
+        self._k = kernels
+        self.device = torch.device(device)
+        self.block_size = block_size
+        self.gpu_cache = [alloc_gpu_cache_layer(num_gpu_blocks, num_kv_heads, head_size, block_size, dtype, self.device)
+                          for _ in range(num_layers)]                                      # :117-121
+        x = cache_x(dtype)
+        self.cpu_cache = [(torch.empty((num_cpu_blocks, num_kv_heads, head_size // x, block_size, x), dtype=dtype,
+                                       pin_memory=num_cpu_blocks > 0),
+                           torch.empty((num_cpu_blocks, num_kv_heads, head_size, block_size), dtype=dtype,
+                                       pin_memory=num_cpu_blocks > 0)) for _ in range(num_layers)]  # :123-133
+        index = self.device.index or 0
+        self.cache_stream = kernels.CudaStream(kernels.CudaStream.LOW_PRI, index)          # :47
+        self.events = [kernels.CudaEvent() for _ in range(num_layers)]                     # :48
+        self.used_events = False
+
+    def get_cache_iface(self):
+        """:53-66.  Returns get(layer) -> (key_cache, value_cache); when a swap was issued this round the
+        calling thread's current stream first waits for that layer's swap to land."""
+        events = self.events if self.used_events else None
+        stream = self._k.CudaStream.current(self.device.index or 0)
+        gpu_cache = self.gpu_cache
+
+        def get(layer_no: int) -> Tuple[torch.Tensor, torch.Tensor]:
+            if events is not None:
+                events[layer_no].wait(stream)
+            return gpu_cache[layer_no]
+
+        return get
+
+    def new_round(self) -> None:
+        self.used_events = False                                                           # :68-70
+
+    def swap_in(self, src_to_dst) -> None:
+        self._swap(self.cpu_cache, self.gpu_cache, src_to_dst)                             # :72-75
+        self.used_events = True
+
+    def swap_out(self, src_to_dst) -> None:
+        self._swap(self.gpu_cache, self.cpu_cache, src_to_dst)                             # :77-80
+        self.used_events = True
+
+    def _swap(self, src, dst, src_to_dst) -> None:
+        """:145-155: every layer's K then V on the cache stream, the layer's event recorded after them."""
+        for i, (src_k, src_v) in enumerate(src):
+            dst_k, dst_v = dst[i]
+            self._k.swap_blocks(src_k, dst_k, src_to_dst, self.cache_stream)
+            self._k.swap_blocks(src_v, dst_v, src_to_dst, self.cache_stream)
+            self.events[i].record(self.cache_stream)
+
+    def copy(self, src_to_dsts) -> None:
+        """:157-169: copy-on-write copies in all layers at once."""
+        self._k.copy_blocks([k for k, _ in self.gpu_cache], [v for _, v in self.gpu_cache], src_to_dsts)
+
+    @staticmethod
+    def get_cache_block_size(block_size: int, num_kv_heads: int, head_size: int, num_layers: int,
+                             dtype: torch.dtype) -> int:
+        return cache_block_bytes(block_size, num_kv_heads, head_size, num_layers, dtype)   # :171-175

@@ -181,3 +181,45 @@ def test_copy_blocks_and_swap_blocks(device):
     assert torch.equal(bits(kd[0][6]), bits(kcs[0][3])) and torch.equal(bits(kd[0][7]), bits(kcs[0][4]))
     with pytest.raises(HipAttnError, match="out of range"):
         K.swap_blocks(kd[0], host, {3: 99})
+
+
+def test_cache_engine_swap_round_trip_and_copy(device):
+    """cache_engine.rs:40-175 end to end: swap blocks out to the host caches and back in on the side
+    stream, the per-layer events ordering the compute stream behind them; copy-on-write copies; sizes."""
+    from aici_amd import paged
+
+    layers, Hkv, d, BS, dt = 3, 2, 64, 16, torch.bfloat16
+    eng = paged.CacheEngine(layers, Hkv, d, BS, dt, num_gpu_blocks=12, num_cpu_blocks=4, device=device)
+    assert eng.gpu_cache[0][0].shape == (12, Hkv, d // 8, BS, 8) and eng.gpu_cache[0][1].shape == (12, Hkv, d, BS)
+    assert eng.cpu_cache[1][0].shape == (4, Hkv, d // 8, BS, 8) and eng.cpu_cache[1][0].is_pinned()
+    assert paged.CacheEngine.get_cache_block_size(BS, Hkv, d, layers, dt) == 2 * BS * Hkv * d * 2 * layers
+    g = torch.Generator().manual_seed(9)
+    want = []
+    for k, v in eng.gpu_cache:
+        kc = torch.randn(k.shape, generator=g).to(dt)
+        vc = torch.randn(v.shape, generator=g).to(dt)
+        k.copy_(kc)
+        v.copy_(vc)
+        want.append((kc, vc))
+    torch.cuda.synchronize()
+    get = eng.get_cache_iface()          # no swap issued yet: plain access
+    assert get(1)[0] is eng.gpu_cache[1][0]
+    eng.swap_out({3: 0, 7: 2})
+    eng.swap_in({0: 10, 2: 11})
+    get = eng.get_cache_iface()          # waits for each layer's swap on the current stream
+    for l in range(layers):
+        k, v = get(l)
+        kk, vv = k.clone(), v.clone()    # ordered behind the layer's event on the current stream
+        torch.cuda.synchronize()
+        assert torch.equal(bits(kk[10]), bits(want[l][0][3])) and torch.equal(bits(kk[11]), bits(want[l][0][7]))
+        assert torch.equal(bits(vv[10]), bits(want[l][1][3])) and torch.equal(bits(vv[11]), bits(want[l][1][7]))
+        assert torch.equal(bits(eng.cpu_cache[l][0][0]), bits(want[l][0][3]))
+        assert torch.equal(bits(kk[:10]), bits(want[l][0][:10]))
+    eng.new_round()
+    assert eng.used_events is False
+    eng.copy({3: [0, 1], 7: [2]})
+    torch.cuda.synchronize()
+    for l in range(layers):
+        k, v = eng.gpu_cache[l]
+        assert torch.equal(bits(k[0]), bits(want[l][0][3])) and torch.equal(bits(k[1]), bits(want[l][0][3]))
+        assert torch.equal(bits(v[2]), bits(want[l][1][7]))
