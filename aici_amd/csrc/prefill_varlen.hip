@@ -480,7 +480,10 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   int kmax = p.causal ? min(Lk, wg_last_row + off + 1) : Lk;
   if (kmax < 0) kmax = 0;
   const int n_tiles = (kmax + BN - 1) / BN;
-  const int wave_row0 = wg_row0 + wave * 32;
+  // Wavefronts w and w + 4 share a SIMD.  Under the causal mask a wavefront's work grows with its rows'
+  // position in the block, so the two of a SIMD take row groups (w, 7 - w): every SIMD gets the same sum.
+  const int row_group = wave < 4 ? wave : 11 - wave;
+  const int wave_row0 = wg_row0 + row_group * 32;
   const int wave_last_row = wave_row0 + 31;
 
   const T *qp = static_cast<const T *>(p.q) + (int64_t)q_begin * p.q_row + (int64_t)h * p.q_head;
