@@ -861,26 +861,38 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   }
 
   // ---- epilogue ---------------------------------------------------------------
+  // The accumulators hold O^T: a lane has 4 consecutive head elements of one row per register quad,
+  // which stored directly would be 16-byte pieces of 32 rows per instruction.  Each wavefront turns
+  // its 32 x d tile through a private piece of LDS (the tiles are dead: every wavefront is past the
+  // last barrier) and writes whole rows, 16 bytes per lane.
   T *op = static_cast<T *>(p.out) + (int64_t)q_begin * p.o_row + (int64_t)h * p.o_head;
-  const int row = wave_row0 + c;
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-  if (row >= Lq) return;
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+  constexpr int OSTR = HDP + 8;  // row pitch of the turned tile, elements
+  T *ost = smem + wave * (32 * OSTR);
 #pragma unroll
   for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
     for (int a = 0; a < 4; a++) {
       const int dcol = dt * 32 + a * 8 + g * 4;
-      if (dcol < p.d) {
-        T r[4];
+      T r[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) r[i] = from_float<T>(acc[dt][a * 4 + i] * inv);
-        *reinterpret_cast<u32x2_t *>(op + (int64_t)row * p.o_row + dcol) = *reinterpret_cast<u32x2_t *>(r);
-      }
+      for (int i = 0; i < 4; i++) r[i] = from_float<T>(acc[dt][a * 4 + i] * inv);
+      *reinterpret_cast<u32x2_t *>(ost + c * OSTR + dcol) = *reinterpret_cast<u32x2_t *>(r);
     }
-  if (p.lse != nullptr && g == 0) {
+  constexpr int CPRO = HDP / 8;  // 16-byte chunks per row
+#pragma unroll
+  for (int it = 0; it < (32 * CPRO + 63) / 64; it++) {
+    const int idx = it * 64 + lane;
+    const int r = idx / CPRO, ch = idx % CPRO;
+    const int row = wave_row0 + r;
+    if (((32 * CPRO) % 64 == 0 || r < 32) && row < Lq && ch < d_chunks)
+      *reinterpret_cast<u32x4_t *>(op + (int64_t)row * p.o_row + ch * 8) =
+          *reinterpret_cast<const u32x4_t *>(ost + r * OSTR + ch * 8);
+  }
+  if (p.lse != nullptr && g == 0 && wave_row0 + c < Lq) {
     const float lse = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : INFINITY;
-    p.lse[((int64_t)b * p.Hq + h) * p.lse_pitch + row] = lse;
+    p.lse[((int64_t)b * p.Hq + h) * p.lse_pitch + wave_row0 + c] = lse;
   }
 }
 
