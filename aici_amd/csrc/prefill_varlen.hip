@@ -870,20 +870,25 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
   constexpr int OSTR = HDP + 8;  // row pitch of the turned tile, elements
   T *ost = smem + wave * (32 * OSTR);
+  // The lane number passes through an empty asm: the addresses below are then computed here, after the
+  // tile loop, instead of before it (where they would have to be kept, and spilled, across the loop).
+  int lane_e = lane;
+  asm volatile("" : "+v"(lane_e));
+  const int c_e = lane_e & 31, g_e = lane_e >> 5;
 #pragma unroll
   for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
     for (int a = 0; a < 4; a++) {
-      const int dcol = dt * 32 + a * 8 + g * 4;
+      const int dcol = dt * 32 + a * 8 + g_e * 4;
       T r[4];
 #pragma unroll
       for (int i = 0; i < 4; i++) r[i] = from_float<T>(acc[dt][a * 4 + i] * inv);
-      *reinterpret_cast<u32x2_t *>(ost + c * OSTR + dcol) = *reinterpret_cast<u32x2_t *>(r);
+      *reinterpret_cast<u32x2_t *>(ost + c_e * OSTR + dcol) = *reinterpret_cast<u32x2_t *>(r);
     }
   constexpr int CPRO = HDP / 8;  // 16-byte chunks per row
 #pragma unroll
   for (int it = 0; it < (32 * CPRO + 63) / 64; it++) {
-    const int idx = it * 64 + lane;
+    const int idx = it * 64 + lane_e;
     const int r = idx / CPRO, ch = idx % CPRO;
     const int row = wave_row0 + r;
     if (((32 * CPRO) % 64 == 0 || r < 32) && row < Lq && ch < d_chunks)
