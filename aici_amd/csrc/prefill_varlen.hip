@@ -869,12 +869,14 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
   constexpr int OSTR = HDP + 8;  // row pitch of the turned tile, elements
-  T *ost = smem + wave * (32 * OSTR);
-  // The lane number passes through an empty asm: the addresses below are then computed here, after the
+  // The thread number passes through an empty asm: the addresses below are then computed here, after the
   // tile loop, instead of before it (where they would have to be kept, and spilled, across the loop).
-  int lane_e = lane;
-  asm volatile("" : "+v"(lane_e));
+  int tid_e = tid;
+  asm volatile("" : "+v"(tid_e));
+  const int lane_e = tid_e & 63, wave_e = tid_e >> 6;
   const int c_e = lane_e & 31, g_e = lane_e >> 5;
+  const int wave_row0_e = wg_row0 + (wave_e < 4 ? wave_e : 11 - wave_e) * 32;
+  T *ost = smem + wave_e * (32 * OSTR);
 #pragma unroll
   for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
@@ -890,14 +892,14 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   for (int it = 0; it < (32 * CPRO + 63) / 64; it++) {
     const int idx = it * 64 + lane_e;
     const int r = idx / CPRO, ch = idx % CPRO;
-    const int row = wave_row0 + r;
+    const int row = wave_row0_e + r;
     if (((32 * CPRO) % 64 == 0 || r < 32) && row < Lq && ch < d_chunks)
       *reinterpret_cast<u32x4_t *>(op + (int64_t)row * p.o_row + ch * 8) =
           *reinterpret_cast<const u32x4_t *>(ost + r * OSTR + ch * 8);
   }
-  if (p.lse != nullptr && g == 0 && wave_row0 + c < Lq) {
+  if (p.lse != nullptr && g_e == 0 && wave_row0_e + c_e < Lq) {
     const float lse = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : INFINITY;
-    p.lse[((int64_t)b * p.Hq + h) * p.lse_pitch + wave_row0 + c] = lse;
+    p.lse[((int64_t)b * p.Hq + h) * p.lse_pitch + wave_row0_e + c_e] = lse;
   }
 }
 
