@@ -491,17 +491,47 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   const T *vp = static_cast<const T *>(p.v) + (PAGED ? (int64_t)kvh * p.vc_head : (int64_t)k_begin * p.v_row + (int64_t)kvh * p.v_head);
   const int d_chunks = p.d / 8;
 
+  // Q operands: lane (g, c) holds q[row c][16 ks + 8 g .. + 8] for every contraction step ks.  Read in
+  // that shape an instruction touches 32 bytes of 32 rows; instead the rows are read whole (16 lanes x
+  // 16 bytes per row, 4 rows per instruction) and turned through a private piece of LDS buffers 1 and 2,
+  // which no tile reaches before the first barrier.
+  constexpr int QSTR = HDP + 8;  // row pitch of the turned Q tile, elements
+  constexpr bool Q_VIA_LDS = (size_t)8 * 32 * QSTR <= (size_t)2 * TL::STAGE_ELEMS;
   vec8 qreg[KSTEPS];
-  {
-    const int row = min(wave_row0 + c, Lq - 1);
+  auto load_q = [&]() {
+    if constexpr (Q_VIA_LDS) {
+      constexpr int CPRQ = HDP / 8;
+      constexpr int NQL = (32 * CPRQ + 63) / 64;
+      T *qst = smem + TL::STAGE_ELEMS + wave * (32 * QSTR);
+      u32x4_t raw[NQL];
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) {
-      u32x4_t raw = {0u, 0u, 0u, 0u};
-      const int ch = 2 * ks + g;
-      if (ch < d_chunks) raw = *reinterpret_cast<const u32x4_t *>(qp + (int64_t)row * p.q_row + ch * 8);
-      qreg[ks] = bit_cast<vec8>(raw);
+      for (int it = 0; it < NQL; it++) {
+        const int idx = min(it * 64 + lane, 32 * CPRQ - 1);
+        const int r = idx / CPRQ, ch = idx % CPRQ;
+        const int row = min(wave_row0 + r, Lq - 1);
+        raw[it] = u32x4_t{0u, 0u, 0u, 0u};
+        if (ch < d_chunks) raw[it] = *reinterpret_cast<const u32x4_t *>(qp + (int64_t)row * p.q_row + ch * 8);
+      }
+#pragma unroll
+      for (int it = 0; it < NQL; it++) {
+        const int idx = it * 64 + lane;
+        if ((32 * CPRQ) % 64 == 0 || idx < 32 * CPRQ)
+          *reinterpret_cast<u32x4_t *>(qst + (idx / CPRQ) * QSTR + (idx % CPRQ) * 8) = raw[it];
+      }
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++)
+        qreg[ks] = *reinterpret_cast<const vec8 *>(qst + c * QSTR + (2 * ks + g) * 8);
+    } else {
+      const int row = min(wave_row0 + c, Lq - 1);
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        u32x4_t raw = {0u, 0u, 0u, 0u};
+        const int ch = 2 * ks + g;
+        if (ch < d_chunks) raw = *reinterpret_cast<const u32x4_t *>(qp + (int64_t)row * p.q_row + ch * 8);
+        qreg[ks] = bit_cast<vec8>(raw);
+      }
     }
-  }
+  };
   f32x16_t acc[NDT];
 #pragma unroll
   for (int dt = 0; dt < NDT; dt++)
@@ -676,8 +706,9 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       store_tile_rows(stage);
   };
 
+  if (n_tiles > 0) load_tile(0);
+  load_q();
   if (n_tiles > 0) {
-    load_tile(0);
     store_tile(0);
     if (n_tiles > 1) load_tile(1);
   }
