@@ -121,6 +121,9 @@ _ERR_FUNCS = {
     "hipattn_block_allocator_trim": [c_void_p, c_int64, c_int64],
     "hipattn_block_allocator_delete": [c_void_p, c_int64],
     "hipattn_block_allocator_get_block_idxes": [c_void_p, c_int64, c_int64, POINTER(c_int64)],
+    "hipattn_block_allocator_swap_out": [c_void_p, c_int64, POINTER(c_int64), c_int64, POINTER(c_int64)],
+    "hipattn_block_allocator_swap_in": [c_void_p, c_int64, POINTER(c_int64), c_int64, POINTER(c_int64), c_int64,
+                                        POINTER(c_int64)],
     "hipattn_batch_builder_new": [c_int64, c_int64, c_int, POINTER(c_void_p)],
     "hipattn_batch_builder_add": [c_void_p, c_int64, POINTER(c_int64), POINTER(c_int32), c_int64, POINTER(c_int64),
                                   c_int64],

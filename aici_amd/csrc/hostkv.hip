@@ -231,6 +231,56 @@ extern "C" char *hipattn_block_allocator_get_block_idxes(const hipattn_block_all
   });
 }
 
+// blocks.rs:176-189 `swap_out`: the sequence's physical blocks, in logical order, which are then
+// released here (trim to 0).  n_out receives the count; out_blocks may be NULL to query it.
+extern "C" char *hipattn_block_allocator_swap_out(hipattn_block_allocator *a, int64_t seq_id, int64_t *out_blocks,
+                                                  int64_t capacity, int64_t *n_out) {
+  HA_PROTECT({
+    HA_CHECK(a != nullptr && n_out != nullptr, "swap_out: allocator or n_out is NULL");
+    auto it = a->seq_blocks.find(seq_id);
+    const int64_t n = it == a->seq_blocks.end() ? 0 : (int64_t)it->second.size();
+    *n_out = n;
+    if (out_blocks == nullptr) return nullptr;  // size query: nothing released
+    HA_CHECK(capacity >= n, "swap_out: room for %lld blocks, sequence %lld holds %lld", (long long)capacity,
+             (long long)seq_id, (long long)n);
+    for (int64_t i = 0; i < n; i++) out_blocks[i] = it->second[(size_t)i];
+    a->trim(seq_id, 0);
+  });
+}
+
+// blocks.rs:191-210 `swap_in`: gives the sequence one block of this allocator per entry of
+// block_idxs (blocks of the other side).  `mapping` (pairs other-side block -> this-side block,
+// n_pairs in use of at most pair_capacity) is shared by the sequences of a group: a block already
+// mapped is forked instead of allocated again, new pairs are appended.
+extern "C" char *hipattn_block_allocator_swap_in(hipattn_block_allocator *a, int64_t seq_id, const int64_t *block_idxs,
+                                                 int64_t n, int64_t *mapping, int64_t pair_capacity, int64_t *n_pairs) {
+  HA_PROTECT({
+    HA_CHECK(a != nullptr && n_pairs != nullptr && (n == 0 || block_idxs != nullptr), "swap_in: bad arguments");
+    HA_CHECK(a->seq_blocks.find(seq_id) == a->seq_blocks.end(), "swap_in: sequence %lld already holds blocks here",
+             (long long)seq_id);
+    HA_CHECK(*n_pairs >= 0 && *n_pairs <= pair_capacity && (pair_capacity == 0 || mapping != nullptr),
+             "swap_in: bad mapping buffer");
+    std::vector<int64_t> v;
+    v.reserve((size_t)n);
+    for (int64_t i = 0; i < n; i++) {
+      int64_t found = -1;
+      for (int64_t k = 0; k < *n_pairs; k++)
+        if (mapping[2 * k] == block_idxs[i]) found = mapping[2 * k + 1];
+      if (found >= 0) {
+        v.push_back(a->fork(found));
+      } else {
+        HA_CHECK(*n_pairs < pair_capacity, "swap_in: mapping buffer full (%lld pairs)", (long long)pair_capacity);
+        const int64_t b2 = a->allocate();
+        mapping[2 * *n_pairs] = block_idxs[i];
+        mapping[2 * *n_pairs + 1] = b2;
+        ++*n_pairs;
+        v.push_back(b2);
+      }
+    }
+    if (!v.empty()) a->seq_blocks[seq_id] = std::move(v);
+  });
+}
+
 extern "C" char *hipattn_batch_builder_new(int64_t block_size, int64_t max_model_len, int paged_attn_kernel_v,
                                            hipattn_batch_builder **outp) {
   HA_PROTECT({

@@ -77,6 +77,106 @@ class BlockAllocator:
              out.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)))
         return out
 
+    def swap_out(self, seq_id: int) -> List[int]:
+        """blocks.rs:176-189: the sequence's blocks (logical order), released here."""
+        n = ctypes.c_int64()
+        call("hipattn_block_allocator_swap_out", self._h, int(seq_id), None, 0, ctypes.byref(n))
+        buf = (ctypes.c_int64 * max(1, n.value))()
+        call("hipattn_block_allocator_swap_out", self._h, int(seq_id), buf, n.value, ctypes.byref(n))
+        return [int(buf[i]) for i in range(n.value)]
+
+    def swap_in(self, seq_id: int, block_idxs: Sequence[int], mapping: dict) -> None:
+        """blocks.rs:191-210: one block here per entry of block_idxs (blocks of the other allocator);
+        `mapping` (other-side block -> block here) is shared by the sequences of a group and extended."""
+        n = len(block_idxs)
+        src = (ctypes.c_int64 * max(1, n))(*[int(b) for b in block_idxs])
+        cap = len(mapping) + n
+        pairs = (ctypes.c_int64 * max(1, 2 * cap))()
+        for i, (k, v) in enumerate(mapping.items()):
+            pairs[2 * i], pairs[2 * i + 1] = int(k), int(v)
+        used = ctypes.c_int64(len(mapping))
+        call("hipattn_block_allocator_swap_in", self._h, int(seq_id), src, n, pairs, cap, ctypes.byref(used))
+        for i in range(len(mapping), used.value):
+            mapping[int(pairs[2 * i])] = int(pairs[2 * i + 1])
+
+
+class BlockSpaceManager:
+    """blocks.rs:259-380: the mapping between logical and physical blocks on both sides of the swap --
+    a device allocator with its admission watermark and a host allocator.  Sequences are plain ids;
+    a group is a list of ids (the reference's SequenceGroup carries the scheduling phase itself, here
+    the caller says which of the group's sequences are running or swapped)."""
+
+    def __init__(self, block_size: int, num_gpu_blocks: int, num_cpu_blocks: int, watermark: float = 0.01):
+        assert watermark >= 0.0
+        self.gpu_allocator = BlockAllocator(block_size, num_gpu_blocks)
+        self.cpu_allocator = BlockAllocator(block_size, num_cpu_blocks)
+        self.gpu_allocator.set_watermark(watermark)
+        self.watermark_blocks = int(watermark * num_gpu_blocks)
+
+    def can_allocate(self, seq_len: int) -> bool:
+        return self.gpu_allocator.can_allocate(seq_len)                                   # :266-270
+
+    def allocate(self, seq_id: int, seq_len: int) -> None:
+        self.gpu_allocator.alloc_seq(seq_id, seq_len)                                     # :272-276
+
+    def can_append_slot(self, num_running_seqs: int) -> bool:
+        return self.gpu_allocator.can_append_slot(num_running_seqs)                       # :278-282
+
+    def append_slots(self, seq_id: int, num_kv_computed: int, seq_len: int) -> List[Tuple[int, int]]:
+        return self.gpu_allocator.append_slots(seq_id, num_kv_computed, seq_len)          # :284-286
+
+    def num_phys_blocks(self, seq_ids: Sequence[int]) -> int:
+        total = 0                                                                         # :364-379
+        for s in seq_ids:
+            n = self.gpu_allocator.num_allocated_blocks(s)
+            if n == 0:
+                n = self.cpu_allocator.num_allocated_blocks(s)
+            else:
+                assert self.cpu_allocator.num_allocated_blocks(s) == 0
+            total += n
+        return total
+
+    def can_swap_in(self, seq_ids: Sequence[int], num_swapped_seqs: Optional[int] = None) -> bool:
+        n = len(seq_ids) if num_swapped_seqs is None else num_swapped_seqs               # :288-293
+        need = self.num_phys_blocks(seq_ids) + n + self.watermark_blocks
+        return self.gpu_allocator.get_num_free_blocks() >= need
+
+    def swap_in(self, swapped_seq_ids: Sequence[int]) -> dict:
+        """:295-305.  Returns host block -> device block for `CacheEngine.swap_in`."""
+        mapping: dict = {}
+        for s in swapped_seq_ids:
+            self.gpu_allocator.swap_in(s, self.cpu_allocator.swap_out(s), mapping)
+        return mapping
+
+    def can_swap_out(self, seq_ids: Sequence[int]) -> bool:
+        return self.num_phys_blocks(seq_ids) <= self.cpu_allocator.get_num_free_blocks()  # :319-322
+
+    def swap_out(self, running_seq_ids: Sequence[int]) -> dict:
+        """:307-317.  Returns device block -> host block for `CacheEngine.swap_out`."""
+        mapping: dict = {}
+        for s in running_seq_ids:
+            self.cpu_allocator.swap_in(s, self.gpu_allocator.swap_out(s), mapping)
+        return mapping
+
+    def get_num_free_gpu_blocks(self) -> int:
+        return self.gpu_allocator.get_num_free_blocks()
+
+    def get_num_free_cpu_blocks(self) -> int:
+        return self.cpu_allocator.get_num_free_blocks()
+
+    # TchSeqMgr (blocks.rs:382-443): fork / trim / delete act on both sides
+    def copy(self, src: int, dst: int, length: int) -> None:
+        self.cpu_allocator.copy(src, dst, length)
+        self.gpu_allocator.copy(src, dst, length)
+
+    def trim(self, seq_id: int, length: int) -> None:
+        self.cpu_allocator.trim(seq_id, length)
+        self.gpu_allocator.trim(seq_id, length)
+
+    def delete(self, seq_id: int) -> None:
+        self.cpu_allocator.delete(seq_id)
+        self.gpu_allocator.delete(seq_id)
+
 
 @dataclass
 class BatchInfo:

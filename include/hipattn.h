@@ -348,6 +348,22 @@ char *hipattn_block_allocator_get_block_idxes(const hipattn_block_allocator *a,
                                               int64_t seq_id, int64_t len,
                                               int64_t *out_slots);
 
+/* blocks.rs:176-189 `swap_out`: copies the sequence's physical block numbers
+ * (logical order) to out_blocks and releases them.  With out_blocks == NULL
+ * only *n_out is set (nothing is released).
+ * blocks.rs:191-210 `swap_in`: one block of this allocator per entry of
+ * block_idxs (blocks of the other allocator); `mapping` holds *n_pairs pairs
+ * (other-side block, this-side block) and is shared by the sequences of a
+ * group: an already mapped block is forked, new pairs are appended. */
+char *hipattn_block_allocator_swap_out(hipattn_block_allocator *a,
+                                       int64_t seq_id, int64_t *out_blocks,
+                                       int64_t capacity, int64_t *n_out);
+char *hipattn_block_allocator_swap_in(hipattn_block_allocator *a,
+                                      int64_t seq_id,
+                                      const int64_t *block_idxs, int64_t n,
+                                      int64_t *mapping, int64_t pair_capacity,
+                                      int64_t *n_pairs);
+
 /* Admission policy of `BlockSpaceManager` over the GPU allocator
  * (blocks.rs:260-283, 321-343): `watermark_blocks = (watermark * num_blocks) as
  * usize` blocks are held back from new sequences so that running ones can keep

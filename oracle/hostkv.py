@@ -118,6 +118,24 @@ class BlockAllocator:
         blocks = self.seq_blocks[seq]
         return [blocks[k // bs] * bs + k % bs for k in range(length)]
 
+    def swap_out(self, seq: int) -> List[int]:                   # blocks.rs:176-189
+        r = list(self.seq_blocks.get(seq, []))
+        self.trim(seq, 0)
+        return r
+
+    def swap_in(self, seq: int, block_idxs: Sequence[int], mapping: dict) -> None:   # blocks.rs:191-210
+        assert self.num_allocated_blocks(seq) == 0
+        v = []
+        for b in block_idxs:
+            if b in mapping:
+                v.append(self._fork(mapping[b]))
+            else:
+                b2 = self._allocate()
+                mapping[b] = b2
+                v.append(b2)
+        if v:
+            self.seq_blocks[seq] = v
+
 
 def build_batch(entries: Sequence[dict], block_size: int, max_model_len: int, paged_attn_kernel_v: int) -> dict:
     """`BatchInfoBuilder::finish` (batch_info.rs:196-315).  Each entry is

@@ -223,3 +223,51 @@ def test_cache_engine_swap_round_trip_and_copy(device):
         k, v = eng.gpu_cache[l]
         assert torch.equal(bits(k[0]), bits(want[l][0][3])) and torch.equal(bits(k[1]), bits(want[l][0][3]))
         assert torch.equal(bits(v[2]), bits(want[l][1][7]))
+
+
+def test_swapped_out_sequence_decodes_the_same_after_swap_in(device):
+    """BlockSpaceManager + CacheEngine together (scheduler.rs preemption by swapping): a sequence's
+    blocks go to the host caches, its device blocks are reused by another sequence, it comes back into
+    different blocks, and paged attention over it gives the same bits as before."""
+    from aici_amd import paged
+
+    Hq, Hkv, d, BS, dt = 8, 2, 64, 16, torch.float16
+    g = torch.Generator().manual_seed(77)
+    mgr = paged.BlockSpaceManager(BS, 12, 8, watermark=0.0)
+    eng = paged.CacheEngine(1, Hkv, d, BS, dt, num_gpu_blocks=12, num_cpu_blocks=8, device=device)
+    kc, vc = eng.gpu_cache[0]
+    kc.zero_()
+    vc.zero_()
+    ctx = 5 * BS + 3
+    mgr.allocate(1, ctx)
+    k = torch.randn((ctx, Hkv, d), generator=g).to(dt).to(device)
+    v = torch.randn((ctx, Hkv, d), generator=g).to(dt).to(device)
+    slots = torch.from_numpy(mgr.gpu_allocator.get_block_idxes(1, ctx)).to(device)
+    K.reshape_and_cache(k, v, kc, vc, slots)
+    q = torch.randn((1, Hq, d), generator=g).to(dt).to(device)
+
+    def decode():
+        blocks = mgr.gpu_allocator.get_block_idxes(1, ctx)[::BS] // BS
+        tables = torch.tensor([blocks.tolist()], dtype=torch.int32, device=device)
+        out = torch.empty_like(q)
+        K.paged_attention_v1(out, q, kc, vc, Hkv, d ** -0.5, tables, torch.tensor([ctx], dtype=torch.int32, device=device),
+                             BS, ctx)
+        return out.cpu(), blocks.tolist()
+
+    before, blocks_before = decode()
+    assert mgr.can_swap_out([1])
+    eng.swap_out(mgr.swap_out([1]))
+    torch.cuda.synchronize()
+    mgr.allocate(2, 4 * BS)                                  # takes some of the blocks sequence 1 had
+    taken = mgr.gpu_allocator.get_block_idxes(2, 4 * BS)
+    K.reshape_and_cache(torch.ones((4 * BS, Hkv, d), dtype=dt, device=device), torch.ones((4 * BS, Hkv, d), dtype=dt, device=device),
+                        kc, vc, torch.from_numpy(taken).to(device))
+    assert set((taken[::BS] // BS).tolist()) & set(blocks_before)
+    assert mgr.can_swap_in([1])
+    eng.new_round()
+    eng.swap_in(mgr.swap_in([1]))
+    kc2, vc2 = eng.get_cache_iface()(0)                      # orders the current stream behind the swap
+    assert kc2 is kc
+    after, blocks_after = decode()
+    assert blocks_after != blocks_before
+    assert torch.equal(bits(after), bits(before))

@@ -228,3 +228,59 @@ def test_multi_entry_block_tables_extension():
     b2 = paged.BatchInfoBuilder(16, 4096, 1)
     b2.add_entry(9, [0, 1, 2], [5, 6, 7], [32, 34, 33])                    # slots out of order
     assert b2.finish().multi_block_tables is None
+
+
+def test_swap_out_and_in_hand_case_with_shared_blocks():
+    """blocks.rs:176-210: swap_out hands over a sequence's blocks and releases them; swap_in on the
+    other side allocates one block per distinct source block -- a block that two sequences of a group
+    share (a fork) is allocated once and forked for the second."""
+    for A in (paged.BlockAllocator, ref.BlockAllocator):
+        gpu, cpu = A(16, 8), A(16, 6)
+        gpu.alloc_seq(1, 40)                     # blocks 0, 1, 2
+        gpu.copy(1, 2, 32)                       # seq 2 shares blocks 0, 1
+        assert gpu.get_num_free_blocks() == 5
+        mapping = {}
+        b1 = gpu.swap_out(1)
+        assert list(b1) == [0, 1, 2] and gpu.num_allocated_blocks(1) == 0
+        assert gpu.get_num_free_blocks() == 6    # 0 and 1 are still held by seq 2
+        cpu.swap_in(1, b1, mapping)
+        assert mapping == {0: 0, 1: 1, 2: 2}
+        b2 = gpu.swap_out(2)
+        assert list(b2) == [0, 1] and gpu.get_num_free_blocks() == 8
+        cpu.swap_in(2, b2, mapping)              # both blocks already mapped: forked, nothing allocated
+        assert mapping == {0: 0, 1: 1, 2: 2} and cpu.get_num_free_blocks() == 3
+        assert list(cpu.get_block_idxes(2, 32)) == list(range(32))
+        cpu.delete(1)
+        assert cpu.get_num_free_blocks() == 4    # block 2 came back; 0 and 1 are still seq 2's
+        assert list(gpu.swap_out(7)) == []       # unknown sequence: nothing to hand over
+        gpu.swap_in(7, [], {})
+        assert gpu.num_allocated_blocks(7) == 0
+
+
+def test_block_space_manager_admission_and_swaps():
+    """blocks.rs:259-380 on 1 % of 300 = 3 watermark blocks."""
+    m = paged.BlockSpaceManager(16, 300, 10, watermark=0.01)
+    assert m.watermark_blocks == 3
+    assert m.can_allocate(297 * 16) and not m.can_allocate(297 * 16 + 1)
+    m.allocate(1, 5 * 16)
+    m.allocate(2, 3 * 16 + 1)
+    m.copy(2, 3, 3 * 16 + 1)                     # seq 3 forks seq 2's four blocks
+    assert m.get_num_free_gpu_blocks() == 291 and m.num_phys_blocks([1, 2, 3]) == 13
+    assert m.can_swap_out([2, 3]) and not m.can_swap_out([1, 2, 3])      # 8 <= 10 < 13
+    to_host = m.swap_out([2, 3])
+    assert to_host == {5: 0, 6: 1, 7: 2, 8: 3}                           # shared blocks travel once
+    assert m.get_num_free_gpu_blocks() == 295 and m.get_num_free_cpu_blocks() == 6
+    assert m.num_phys_blocks([2, 3]) == 8                                # now counted on the host side
+    assert m.can_swap_in([2, 3])                                         # 8 + 2 + 3 <= 295
+    to_dev = m.swap_in([2, 3])
+    # the free list is a stack: the blocks that came back last go out first
+    assert sorted(to_dev) == [0, 1, 2, 3] and len(set(to_dev.values())) == 4
+    assert m.get_num_free_cpu_blocks() == 10 and m.get_num_free_gpu_blocks() == 291
+    assert list(m.gpu_allocator.get_block_idxes(2, 49)) == list(m.gpu_allocator.get_block_idxes(3, 49))
+    assert m.can_append_slot(291) and not m.can_append_slot(292)
+    pairs = m.append_slots(3, 49, 50)            # seq 3 writes into the shared last block: copy-on-write
+    assert len(pairs) == 1 and pairs[0][0] == to_dev[3]
+    m.delete(2)
+    m.delete(3)
+    m.trim(1, 16)
+    assert m.get_num_free_gpu_blocks() == 299
