@@ -198,9 +198,9 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
   constexpr int X = 8;
   constexpr int KP = 72;  // K slab row pitch in elements: 8 chunks + 16 bytes, keeps the transposed 16-byte reads apart
   constexpr int VP = 64;  // V slab row pitch: the 2-byte column accesses of a wavefront fall in one row
-  __shared__ __attribute__((aligned(16))) E slab[4][8 * KP + 8 * VP];
+  __shared__ __attribute__((aligned(16))) E slab[4][16 * KP + 16 * VP];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  E *ks = slab[wave], *vs = slab[wave] + 8 * KP;
+  E *ks = slab[wave], *vs = slab[wave] + 16 * KP;
   const int64_t wg_t0 = (int64_t)blockIdx.x * 16;
   const int chunks_per_head = g.head_size / X;
   const int groups_per_head = chunks_per_head / 8;
@@ -221,6 +221,44 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
     }
   }
   const int hi = lane >> 3, lo = lane & 7;
+  // A workgroup whose 16 tokens fill one whole block: a tile is then 16 tokens deep and every store
+  // instruction writes whole rows of the cache -- K as 256-byte [chunk][16 tokens] rows, V as the
+  // 32-byte [16 tokens] rows of 32 consecutive head elements, 1 KiB contiguous either way.
+  if (SCATTER && g.block_size == 16 && run_slot[0] >= 0 && run_slot[0] % 16 == 0 && run_slot[1] == run_slot[0] + 8) {
+    const int64_t blk = run_slot[0] / 16;
+    for (int item = wave; item < items_per_half; item += 4) {
+      const int h = item / groups_per_head, cg = item % groups_per_head;
+      E *kc_base = key_cache + blk * g.k_block_stride + h * g.k_head_stride;
+      E *vc_base = value_cache + blk * g.v_block_stride + h * g.v_head_stride;
+#pragma unroll
+      for (int half = 0; half < 2; half++) {  // tokens hi and hi + 8, chunk lo
+        const E *k_tok = key + (wg_t0 + 8 * half + hi) * key_tok_stride + h * key_head_stride + (cg * 8 + lo) * X;
+        const E *v_tok = value + (wg_t0 + 8 * half + hi) * val_tok_stride + h * val_head_stride + (cg * 8 + lo) * X;
+        *reinterpret_cast<uint4 *>(ks + (8 * half + hi) * KP + lo * X) = *reinterpret_cast<const uint4 *>(k_tok);
+        *reinterpret_cast<uint4 *>(vs + (8 * half + hi) * VP + lo * X) = *reinterpret_cast<const uint4 *>(v_tok);
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the slab is private to this wavefront
+      const int tok = lane & 15, c4 = lane >> 4;
+#pragma unroll
+      for (int i = 0; i < 2; i++) {  // chunk rows 4i + c4: 4 rows x 256 bytes per instruction
+        const int c = 4 * i + c4;
+        *reinterpret_cast<uint4 *>(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X) =
+            *reinterpret_cast<const uint4 *>(ks + tok * KP + c * X);
+      }
+      const int th = lane & 1;  // which 8 tokens of the row
+#pragma unroll
+      for (int i = 0; i < 2; i++) {  // head elements 32i + lane / 2: 32 rows x 32 bytes per instruction
+        const int e = 32 * i + (lane >> 1);
+        uint4 o;
+        E *oe = reinterpret_cast<E *>(&o);
+#pragma unroll
+        for (int t = 0; t < 8; t++) oe[t] = vs[(8 * th + t) * VP + e];
+        *reinterpret_cast<uint4 *>(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th) = o;
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // slab reads done before the next item overwrites it
+    }
+    return;
+  }
   for (int item = wave; item < 2 * items_per_half; item += 4) {  // uniform per wavefront
     const int half = item / items_per_half;
     const int rem = item % items_per_half;
