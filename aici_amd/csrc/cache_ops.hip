@@ -187,7 +187,9 @@ __global__ __launch_bounds__(256) void cache_move_run8_kernel(
 // private LDS slab: it reads the source in the source's order (128-byte runs), transposes in LDS, and
 // writes the destination in the destination's order -- K as 128-byte runs [chunk][8 tokens], V as the 8
 // tokens (16 bytes) of each of the tile's 64 head elements.  16 tokens per workgroup as in the kernel
-// above; groups that are not a run of 8 slots take its per-token path.
+// above; groups that are not a run of 8 slots take its per-token path, and a workgroup whose 16 tokens
+// fill one whole block moves 16-token tiles, whose cache side is whole rows ([chunk][16 tokens] = 256
+// bytes of K, [16 tokens] = 32 bytes of each V element, 1 KiB contiguous per instruction).
 template <typename Slot, bool SCATTER>
 __global__ __launch_bounds__(256) void cache_move_tile_kernel(
     uint16_t *__restrict__ key, uint16_t *__restrict__ value, uint16_t *__restrict__ key_cache,
@@ -221,39 +223,61 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
     }
   }
   const int hi = lane >> 3, lo = lane & 7;
-  // A workgroup whose 16 tokens fill one whole block: a tile is then 16 tokens deep and every store
-  // instruction writes whole rows of the cache -- K as 256-byte [chunk][16 tokens] rows, V as the
-  // 32-byte [16 tokens] rows of 32 consecutive head elements, 1 KiB contiguous either way.
-  if (SCATTER && g.block_size == 16 && run_slot[0] >= 0 && run_slot[0] % 16 == 0 && run_slot[1] == run_slot[0] + 8) {
+  // A workgroup whose 16 tokens fill one whole block: a tile is then 16 tokens deep and every access to
+  // the cache covers whole rows -- K as 256-byte [chunk][16 tokens] rows, V as the 32-byte [16 tokens]
+  // rows of 32 consecutive head elements, 1 KiB contiguous either way.
+  if (g.block_size == 16 && run_slot[0] >= 0 && run_slot[0] % 16 == 0 && run_slot[1] == run_slot[0] + 8) {
     const int64_t blk = run_slot[0] / 16;
     for (int item = wave; item < items_per_half; item += 4) {
       const int h = item / groups_per_head, cg = item % groups_per_head;
       E *kc_base = key_cache + blk * g.k_block_stride + h * g.k_head_stride;
       E *vc_base = value_cache + blk * g.v_block_stride + h * g.v_head_stride;
-#pragma unroll
-      for (int half = 0; half < 2; half++) {  // tokens hi and hi + 8, chunk lo
-        const E *k_tok = key + (wg_t0 + 8 * half + hi) * key_tok_stride + h * key_head_stride + (cg * 8 + lo) * X;
-        const E *v_tok = value + (wg_t0 + 8 * half + hi) * val_tok_stride + h * val_head_stride + (cg * 8 + lo) * X;
-        *reinterpret_cast<uint4 *>(ks + (8 * half + hi) * KP + lo * X) = *reinterpret_cast<const uint4 *>(k_tok);
-        *reinterpret_cast<uint4 *>(vs + (8 * half + hi) * VP + lo * X) = *reinterpret_cast<const uint4 *>(v_tok);
-      }
-      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the slab is private to this wavefront
       const int tok = lane & 15, c4 = lane >> 4;
+      const int th = lane & 1;  // which 8 tokens of a V row
+      if (SCATTER) {
 #pragma unroll
-      for (int i = 0; i < 2; i++) {  // chunk rows 4i + c4: 4 rows x 256 bytes per instruction
-        const int c = 4 * i + c4;
-        *reinterpret_cast<uint4 *>(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X) =
-            *reinterpret_cast<const uint4 *>(ks + tok * KP + c * X);
-      }
-      const int th = lane & 1;  // which 8 tokens of the row
+        for (int half = 0; half < 2; half++) {  // tokens hi and hi + 8, chunk lo
+          const E *k_tok = key + (wg_t0 + 8 * half + hi) * key_tok_stride + h * key_head_stride + (cg * 8 + lo) * X;
+          const E *v_tok = value + (wg_t0 + 8 * half + hi) * val_tok_stride + h * val_head_stride + (cg * 8 + lo) * X;
+          *reinterpret_cast<uint4 *>(ks + (8 * half + hi) * KP + lo * X) = *reinterpret_cast<const uint4 *>(k_tok);
+          *reinterpret_cast<uint4 *>(vs + (8 * half + hi) * VP + lo * X) = *reinterpret_cast<const uint4 *>(v_tok);
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the slab is private to this wavefront
 #pragma unroll
-      for (int i = 0; i < 2; i++) {  // head elements 32i + lane / 2: 32 rows x 32 bytes per instruction
-        const int e = 32 * i + (lane >> 1);
-        uint4 o;
-        E *oe = reinterpret_cast<E *>(&o);
+        for (int i = 0; i < 2; i++) {  // chunk rows 4i + c4: 4 rows x 256 bytes per instruction
+          const int c = 4 * i + c4;
+          *reinterpret_cast<uint4 *>(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X) =
+              *reinterpret_cast<const uint4 *>(ks + tok * KP + c * X);
+        }
 #pragma unroll
-        for (int t = 0; t < 8; t++) oe[t] = vs[(8 * th + t) * VP + e];
-        *reinterpret_cast<uint4 *>(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th) = o;
+        for (int i = 0; i < 2; i++) {  // head elements 32i + lane / 2: 32 rows x 32 bytes per instruction
+          const int e = 32 * i + (lane >> 1);
+          uint4 o;
+          E *oe = reinterpret_cast<E *>(&o);
+#pragma unroll
+          for (int t = 0; t < 8; t++) oe[t] = vs[(8 * th + t) * VP + e];
+          *reinterpret_cast<uint4 *>(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th) = o;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+          const int c = 4 * i + c4;
+          *reinterpret_cast<uint4 *>(ks + tok * KP + c * X) =
+              *reinterpret_cast<const uint4 *>(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X);
+          const int e = 32 * i + (lane >> 1);
+          const uint4 vin = *reinterpret_cast<const uint4 *>(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th);
+          const E *ve = reinterpret_cast<const E *>(&vin);
+#pragma unroll
+          for (int t = 0; t < 8; t++) vs[(8 * th + t) * VP + e] = ve[t];
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+          E *k_tok = key + (wg_t0 + 8 * half + hi) * key_tok_stride + h * key_head_stride + (cg * 8 + lo) * X;
+          E *v_tok = value + (wg_t0 + 8 * half + hi) * val_tok_stride + h * val_head_stride + (cg * 8 + lo) * X;
+          *reinterpret_cast<uint4 *>(k_tok) = *reinterpret_cast<const uint4 *>(ks + (8 * half + hi) * KP + lo * X);
+          *reinterpret_cast<uint4 *>(v_tok) = *reinterpret_cast<const uint4 *>(vs + (8 * half + hi) * VP + lo * X);
+        }
       }
       __builtin_amdgcn_s_waitcnt(0xc07f);  // slab reads done before the next item overwrites it
     }
@@ -406,9 +430,9 @@ void launch_move(const hipattn_tensor *key, const hipattn_tensor *value,
     // long inputs (prompts): 8-token workgroups with the transposing fast path
     if (vec && T >= 1024 && g.block_size % 8 == 0 && aligned16(vc) && g.v_block_stride % 8 == 0 &&
         g.v_head_stride % 8 == 0) {
-      // The LDS-transposing kernel pays off for the scatter (its stores become whole lines) once there are
-      // enough 16-token workgroups to hide its load -> LDS -> store chains; the gather is as fast without it.
-      if (SCATTER && g.head_size % 64 == 0 && T >= 16384 && getenv("HIPATTN_CACHE_MOVE_NO_LDS") == nullptr) {
+      // The LDS-transposing kernel pays off (whole rows on both sides) once there are enough 16-token
+      // workgroups to hide its load -> LDS -> store chains.
+      if (g.head_size % 64 == 0 && T >= 16384 && getenv("HIPATTN_CACHE_MOVE_NO_LDS") == nullptr) {
         cache_move_tile_kernel<Slot, SCATTER><<<dim3((unsigned)((T + 15) / 16)), 256, 0, stream>>>(
             kp, vp, kc, vc, sp, T, key->strides[0], key->strides[1], value->strides[0], value->strides[1], g);
         check_launch(SCATTER ? "reshape_and_cache" : "gather_cached_kv");
