@@ -181,7 +181,8 @@ __global__ __launch_bounds__(256) void cache_move_run8_kernel(
   }
 }
 
-// Coalesced on both sides (2-byte elements, head size a multiple of 64).  The input is token-major,
+// Coalesced on both sides (2-byte elements, head size a multiple of 8; the last group of a head has fewer
+// than 8 chunks when it is not a multiple of 64, and the lanes beyond them sit out).  The input is token-major,
 // the cache chunk-major, so some side of a direct copy always touches 16-byte pieces 256 bytes apart.
 // Here a wavefront moves one (8 tokens) x (8 chunks = 64 head elements) tile of one head through a
 // private LDS slab: it reads the source in the source's order (128-byte runs), transposes in LDS, and
@@ -205,7 +206,7 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
   E *ks = slab[wave], *vs = slab[wave] + 16 * KP;
   const int64_t wg_t0 = (int64_t)blockIdx.x * 16;
   const int chunks_per_head = g.head_size / X;
-  const int groups_per_head = chunks_per_head / 8;
+  const int groups_per_head = (chunks_per_head + 7) / 8;  // the last group of a head may hold fewer than 8 chunks
   const int items_per_half = g.num_heads * groups_per_head;
   int64_t run_slot[2];
 #pragma unroll
@@ -230,6 +231,7 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
     const int64_t blk = run_slot[0] / 16;
     for (int item = wave; item < items_per_half; item += 4) {
       const int h = item / groups_per_head, cg = item % groups_per_head;
+      const int nc = min(8, chunks_per_head - 8 * cg);  // chunks in this group
       E *kc_base = key_cache + blk * g.k_block_stride + h * g.k_head_stride;
       E *vc_base = value_cache + blk * g.v_block_stride + h * g.v_head_stride;
       const int tok = lane & 15, c4 = lane >> 4;
@@ -239,15 +241,18 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
         for (int half = 0; half < 2; half++) {  // tokens hi and hi + 8, chunk lo
           const E *k_tok = key + (wg_t0 + 8 * half + hi) * key_tok_stride + h * key_head_stride + (cg * 8 + lo) * X;
           const E *v_tok = value + (wg_t0 + 8 * half + hi) * val_tok_stride + h * val_head_stride + (cg * 8 + lo) * X;
-          *reinterpret_cast<uint4 *>(ks + (8 * half + hi) * KP + lo * X) = *reinterpret_cast<const uint4 *>(k_tok);
-          *reinterpret_cast<uint4 *>(vs + (8 * half + hi) * VP + lo * X) = *reinterpret_cast<const uint4 *>(v_tok);
+          if (lo < nc) {
+            *reinterpret_cast<uint4 *>(ks + (8 * half + hi) * KP + lo * X) = *reinterpret_cast<const uint4 *>(k_tok);
+            *reinterpret_cast<uint4 *>(vs + (8 * half + hi) * VP + lo * X) = *reinterpret_cast<const uint4 *>(v_tok);
+          }
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the slab is private to this wavefront
 #pragma unroll
         for (int i = 0; i < 2; i++) {  // chunk rows 4i + c4: 4 rows x 256 bytes per instruction
           const int c = 4 * i + c4;
-          *reinterpret_cast<uint4 *>(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X) =
-              *reinterpret_cast<const uint4 *>(ks + tok * KP + c * X);
+          if (c < nc)
+            *reinterpret_cast<uint4 *>(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X) =
+                *reinterpret_cast<const uint4 *>(ks + tok * KP + c * X);
         }
 #pragma unroll
         for (int i = 0; i < 2; i++) {  // head elements 32i + lane / 2: 32 rows x 32 bytes per instruction
@@ -256,27 +261,32 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
           E *oe = reinterpret_cast<E *>(&o);
 #pragma unroll
           for (int t = 0; t < 8; t++) oe[t] = vs[(8 * th + t) * VP + e];
-          *reinterpret_cast<uint4 *>(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th) = o;
+          if (e < nc * X) *reinterpret_cast<uint4 *>(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th) = o;
         }
       } else {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
           const int c = 4 * i + c4;
-          *reinterpret_cast<uint4 *>(ks + tok * KP + c * X) =
-              *reinterpret_cast<const uint4 *>(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X);
+          if (c < nc)
+            *reinterpret_cast<uint4 *>(ks + tok * KP + c * X) =
+                *reinterpret_cast<const uint4 *>(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X);
           const int e = 32 * i + (lane >> 1);
-          const uint4 vin = *reinterpret_cast<const uint4 *>(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th);
-          const E *ve = reinterpret_cast<const E *>(&vin);
+          if (e < nc * X) {
+            const uint4 vin = *reinterpret_cast<const uint4 *>(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th);
+            const E *ve = reinterpret_cast<const E *>(&vin);
 #pragma unroll
-          for (int t = 0; t < 8; t++) vs[(8 * th + t) * VP + e] = ve[t];
+            for (int t = 0; t < 8; t++) vs[(8 * th + t) * VP + e] = ve[t];
+          }
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);
 #pragma unroll
         for (int half = 0; half < 2; half++) {
           E *k_tok = key + (wg_t0 + 8 * half + hi) * key_tok_stride + h * key_head_stride + (cg * 8 + lo) * X;
           E *v_tok = value + (wg_t0 + 8 * half + hi) * val_tok_stride + h * val_head_stride + (cg * 8 + lo) * X;
-          *reinterpret_cast<uint4 *>(k_tok) = *reinterpret_cast<const uint4 *>(ks + (8 * half + hi) * KP + lo * X);
-          *reinterpret_cast<uint4 *>(v_tok) = *reinterpret_cast<const uint4 *>(vs + (8 * half + hi) * VP + lo * X);
+          if (lo < nc) {
+            *reinterpret_cast<uint4 *>(k_tok) = *reinterpret_cast<const uint4 *>(ks + (8 * half + hi) * KP + lo * X);
+            *reinterpret_cast<uint4 *>(v_tok) = *reinterpret_cast<const uint4 *>(vs + (8 * half + hi) * VP + lo * X);
+          }
         }
       }
       __builtin_amdgcn_s_waitcnt(0xc07f);  // slab reads done before the next item overwrites it
@@ -300,25 +310,34 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
       E *v_tok = value + (t0 + hi) * val_tok_stride + h * val_head_stride + (cg * 8 + lo) * X;
       E *k_cache = kc_base + ((int64_t)(cg * 8 + hi) * g.block_size + off0 + lo) * X;
       E *v_cache = vc_base + (int64_t)((cg * 8 + hi) * X + lo) * g.block_size + off0;
+      const int nc = min(8, chunks_per_head - 8 * cg);  // chunks in this group
       if (SCATTER) {
-        *reinterpret_cast<uint4 *>(ks + hi * KP + lo * X) = *reinterpret_cast<const uint4 *>(k_tok);
-        *reinterpret_cast<uint4 *>(vs + hi * VP + lo * X) = *reinterpret_cast<const uint4 *>(v_tok);
+        if (lo < nc) {
+          *reinterpret_cast<uint4 *>(ks + hi * KP + lo * X) = *reinterpret_cast<const uint4 *>(k_tok);
+          *reinterpret_cast<uint4 *>(vs + hi * VP + lo * X) = *reinterpret_cast<const uint4 *>(v_tok);
+        }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the slab is private to this wavefront
-        *reinterpret_cast<uint4 *>(k_cache) = *reinterpret_cast<const uint4 *>(ks + lo * KP + hi * X);
-        uint4 o;
-        E *oe = reinterpret_cast<E *>(&o);
+        if (hi < nc) {
+          *reinterpret_cast<uint4 *>(k_cache) = *reinterpret_cast<const uint4 *>(ks + lo * KP + hi * X);
+          uint4 o;
+          E *oe = reinterpret_cast<E *>(&o);
 #pragma unroll
-        for (int t = 0; t < 8; t++) oe[t] = vs[t * VP + lane];  // element (hi, lo) of token t
-        *reinterpret_cast<uint4 *>(v_cache) = o;
+          for (int t = 0; t < 8; t++) oe[t] = vs[t * VP + lane];  // element (hi, lo) of token t
+          *reinterpret_cast<uint4 *>(v_cache) = o;
+        }
       } else {
-        *reinterpret_cast<uint4 *>(ks + lo * KP + hi * X) = *reinterpret_cast<const uint4 *>(k_cache);
-        const uint4 vin = *reinterpret_cast<const uint4 *>(v_cache);
-        const E *ve = reinterpret_cast<const E *>(&vin);
+        if (hi < nc) {
+          *reinterpret_cast<uint4 *>(ks + lo * KP + hi * X) = *reinterpret_cast<const uint4 *>(k_cache);
+          const uint4 vin = *reinterpret_cast<const uint4 *>(v_cache);
+          const E *ve = reinterpret_cast<const E *>(&vin);
 #pragma unroll
-        for (int t = 0; t < 8; t++) vs[t * VP + lane] = ve[t];
+          for (int t = 0; t < 8; t++) vs[t * VP + lane] = ve[t];
+        }
         __builtin_amdgcn_s_waitcnt(0xc07f);
-        *reinterpret_cast<uint4 *>(k_tok) = *reinterpret_cast<const uint4 *>(ks + hi * KP + lo * X);
-        *reinterpret_cast<uint4 *>(v_tok) = *reinterpret_cast<const uint4 *>(vs + hi * VP + lo * X);
+        if (lo < nc) {
+          *reinterpret_cast<uint4 *>(k_tok) = *reinterpret_cast<const uint4 *>(ks + hi * KP + lo * X);
+          *reinterpret_cast<uint4 *>(v_tok) = *reinterpret_cast<const uint4 *>(vs + hi * VP + lo * X);
+        }
       }
       __builtin_amdgcn_s_waitcnt(0xc07f);  // slab reads done before the next item overwrites it
       continue;
@@ -332,7 +351,7 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
       const int64_t blk = slot / g.block_size;
       if (blk >= g.num_blocks) continue;
       const int off = (int)(slot % g.block_size);
-      if (lane < 8) {
+      if (lane < min(8, chunks_per_head - 8 * cg)) {
         const int c = cg * 8 + lane;
         E *kp = key + token * key_tok_stride + h * key_head_stride + c * X;
         E *vp = value + token * val_tok_stride + h * val_head_stride + c * X;
@@ -432,7 +451,7 @@ void launch_move(const hipattn_tensor *key, const hipattn_tensor *value,
         g.v_head_stride % 8 == 0) {
       // The LDS-transposing kernel pays off (whole rows on both sides) once there are enough 16-token
       // workgroups to hide its load -> LDS -> store chains.
-      if (g.head_size % 64 == 0 && T >= 16384 && getenv("HIPATTN_CACHE_MOVE_NO_LDS") == nullptr) {
+      if (T >= 16384 && getenv("HIPATTN_CACHE_MOVE_NO_LDS") == nullptr) {
         cache_move_tile_kernel<Slot, SCATTER><<<dim3((unsigned)((T + 15) / 16)), 256, 0, stream>>>(
             kp, vp, kc, vc, sp, T, key->strides[0], key->strides[1], value->strides[0], value->strides[1], g);
         check_launch(SCATTER ? "reshape_and_cache" : "gather_cached_kv");

@@ -58,14 +58,16 @@ def test_reshape_and_cache_and_gather_bit_exact(device, dtype, slot_dtype, strid
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("strided", [False, True])
-@pytest.mark.parametrize("d", [96, 128, 64])   # 96: register-tile kernel; multiples of 64: LDS-tile kernel
-def test_long_inputs_runs_of_tokens_mixed_with_everything_else(device, dtype, strided, d):
+@pytest.mark.parametrize("d,first", [(96, 512), (128, 512),      # the register-tile kernel (under 16384 tokens)
+                                     (128, 16000), (64, 16000),   # the LDS-tile kernel
+                                     (96, 16000), (80, 16000)])   # ... with a partial last chunk group per head
+def test_long_inputs_runs_of_tokens_mixed_with_everything_else(device, dtype, strided, d, first):
     """More than 1024 tokens: the kernels move aligned runs of 8 tokens as tiles and fall back per
     token elsewhere.  The slot list mixes prompts that fill permuted blocks in order (lengths not
     multiples of 8, so runs straddle sequences), a prompt that starts in the middle of a block,
     padding slots inside a run, decode-like random slots, a slot past the cache and a ragged tail."""
     g = torch.Generator().manual_seed(7)
-    H, bs, nb = 4, 16, (200 if d == 96 else 1200)
+    H, bs, nb = 4, 16, 1200
     perm = torch.randperm(nb, generator=g).tolist()
     slots = []
 
@@ -74,7 +76,7 @@ def test_long_inputs_runs_of_tokens_mixed_with_everything_else(device, dtype, st
         blocks = [perm.pop() for _ in range(need)]
         slots.extend(blocks[(start_off + t) // bs] * bs + (start_off + t) % bs for t in range(n))
 
-    prompt(512 if d == 96 else 16000)   # d = 64, 128: long enough for the LDS-tile scatter kernel
+    prompt(first)
     prompt(203)
     prompt(77, start_off=5)
     prompt(256)
