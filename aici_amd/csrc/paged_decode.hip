@@ -27,6 +27,7 @@
 // probabilities.
 #include "common.h"
 #include "device_types.h"
+#include "paged_decode_generic.h"
 #include "workspace.h"
 
 namespace hipattn {
@@ -821,6 +822,33 @@ int choose_part_blocks(int64_t S, int Hkv, int col_groups, int max_ctx) {
   return (int)pb;
 }
 
+GenericDecodeParams generic_params(const DecodeParams &p, int head_size, int block_size, float scale) {
+  GenericDecodeParams g;
+  memset(&g, 0, sizeof g);
+  g.q = p.q;
+  g.q_stride = p.q_stride;
+  g.kc = p.kc;
+  g.vc = p.vc;
+  g.k_block_stride = p.k_block_stride;
+  g.k_head_stride = p.k_head_stride;
+  g.v_block_stride = p.v_block_stride;
+  g.v_head_stride = p.v_head_stride;
+  g.num_blocks = p.num_blocks;
+  g.block_tables = p.block_tables;
+  g.table_stride = p.max_blocks;
+  g.context_lens = p.context_lens;
+  g.alibi = p.alibi;
+  g.scale = scale;
+  g.Hq = p.Hq;
+  g.G = p.G;
+  g.head_size = head_size;
+  g.block_size = block_size;
+  g.num_seqs = p.num_seqs;
+  g.out = p.out;
+  g.out_stride = p.out_stride;
+  return g;
+}
+
 void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn_tensor *max_logits,
                           hipattn_tensor *tmp_out, const hipattn_tensor *query, const hipattn_tensor *key_cache,
                           const hipattn_tensor *value_cache, int num_kv_heads, float scale,
@@ -833,13 +861,18 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
   check_tensor(value_cache, "value_cache", 4);
   check_tensor(block_tables, "block_tables", 2);
   check_tensor(context_lens, "context_lens", 1);
-  HA_CHECK(query->dtype == HIPATTN_F16 || query->dtype == HIPATTN_BF16,
-           "%s: unsupported data type %s (supported: f16, bf16)", op, dtype_name(query->dtype));
+  HA_CHECK(is_float_dtype(query->dtype), "%s: unsupported data type %s (supported: f16, bf16, f32)", op,
+           dtype_name(query->dtype));
   HA_CHECK(out->dtype == query->dtype && key_cache->dtype == query->dtype && value_cache->dtype == query->dtype,
            "%s: out, query and caches must share a dtype", op);
   HA_CHECK(block_tables->dtype == HIPATTN_I32 && context_lens->dtype == HIPATTN_I32,
            "%s: block_tables and context_lens must be int32", op);
-  HA_CHECK(block_size == kBlockSize, "%s: unsupported block size %d (supported: %d)", op, block_size, kBlockSize);
+  HA_CHECK(block_size == 8 || block_size == 16 || block_size == 32,
+           "%s: unsupported block size %d (supported: 8, 16, 32)", op, block_size);
+  // The MFMA kernels take 16-token blocks of a 2-byte type (what rLLM runs); the rest of the
+  // reference's support matrix goes to the fp32-FMA kernel.
+  const bool generic = block_size != kBlockSize || query->dtype == HIPATTN_F32;
+  const int x = 16 / dtype_size(query->dtype);
   const int64_t S = query->sizes[0];
   const int Hq = (int)query->sizes[1];
   const int hd = (int)query->sizes[2];
@@ -847,24 +880,29 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
   HA_CHECK(num_kv_heads > 0 && Hq % num_kv_heads == 0, "%s: %d query heads not divisible by %d kv heads", op, Hq,
            num_kv_heads);
   HA_CHECK(key_cache->sizes[1] == num_kv_heads && key_cache->sizes[2] * key_cache->sizes[4] == hd &&
-               key_cache->sizes[3] == block_size && key_cache->sizes[4] == 8,
-           "%s: key_cache shape does not match [nb, %d, %d/8, %d, 8]", op, num_kv_heads, hd, block_size);
+               key_cache->sizes[3] == block_size && key_cache->sizes[4] == x,
+           "%s: key_cache shape does not match [nb, %d, %d/%d, %d, %d]", op, num_kv_heads, hd, x, block_size, x);
   HA_CHECK(value_cache->sizes[0] == key_cache->sizes[0] && value_cache->sizes[1] == num_kv_heads &&
                value_cache->sizes[2] == hd && value_cache->sizes[3] == block_size,
            "%s: value_cache shape does not match [nb, %d, %d, %d]", op, num_kv_heads, hd, block_size);
-  HA_CHECK(key_cache->strides[4] == 1 && key_cache->strides[3] == 8 && key_cache->strides[2] == 8 * block_size &&
+  HA_CHECK(key_cache->strides[4] == 1 && key_cache->strides[3] == x && key_cache->strides[2] == x * block_size &&
                value_cache->strides[3] == 1 && value_cache->strides[2] == block_size,
            "%s: cache inner dims must be contiguous", op);
-  HA_CHECK(key_cache->strides[0] % 8 == 0 && key_cache->strides[1] % 8 == 0 && value_cache->strides[0] % 4 == 0 &&
-               value_cache->strides[1] % 4 == 0,
-           "%s: cache block/head strides must keep 16-byte alignment", op);
-  HA_CHECK((reinterpret_cast<uintptr_t>(key_cache->data) & 15) == 0 &&
-               (reinterpret_cast<uintptr_t>(value_cache->data) & 15) == 0 &&
-               (reinterpret_cast<uintptr_t>(query->data) & 15) == 0 && (reinterpret_cast<uintptr_t>(out->data) & 7) == 0,
-           "%s: tensors must be 16-byte aligned", op);
+  HA_CHECK(key_cache->strides[0] % x == 0 && key_cache->strides[1] % x == 0 &&
+               (reinterpret_cast<uintptr_t>(key_cache->data) & 15) == 0,
+           "%s: key_cache blocks and heads must keep 16-byte alignment", op);
   HA_CHECK((hd <= 1 || (query->strides[2] == 1 && out->strides[2] == 1)) && query->strides[1] == hd &&
-               out->strides[1] == hd && query->strides[0] % 8 == 0 && out->strides[0] % 4 == 0,
-           "%s: query/out heads must be contiguous with an aligned row stride", op);
+               out->strides[1] == hd,
+           "%s: query/out heads must be contiguous", op);
+  if (!generic) {
+    HA_CHECK(value_cache->strides[0] % 4 == 0 && value_cache->strides[1] % 4 == 0,
+             "%s: cache block/head strides must keep 16-byte alignment", op);
+    HA_CHECK((reinterpret_cast<uintptr_t>(value_cache->data) & 15) == 0 &&
+                 (reinterpret_cast<uintptr_t>(query->data) & 15) == 0 && (reinterpret_cast<uintptr_t>(out->data) & 7) == 0,
+             "%s: tensors must be 16-byte aligned", op);
+    HA_CHECK(query->strides[0] % 8 == 0 && out->strides[0] % 4 == 0,
+             "%s: query/out need an aligned row stride", op);
+  }
   HA_CHECK(block_tables->sizes[0] == S && context_lens->sizes[0] == S, "%s: block_tables/context_lens need %lld rows", op,
            (long long)S);
   check_contiguous(context_lens, "context_lens");
@@ -934,6 +972,15 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
     check_data(max_logits, "max_logits");
     check_data(tmp_out, "tmp_out");
     HA_CHECK((reinterpret_cast<uintptr_t>(tmp_out->data) & 7) == 0, "%s: tmp_out must be 8-byte aligned", op);
+    if (generic) {
+      GenericDecodeParams g = generic_params(p, hd, block_size, scale);
+      g.num_parts = (int)P;
+      g.ws_l = static_cast<float *>(exp_sums->data);
+      g.ws_m = static_cast<float *>(max_logits->data);
+      g.tmp_out = tmp_out->data;
+      paged_decode_generic(g, query->dtype, true, max_context_len, stream);
+      return;
+    }
     int64_t pb = (max_blocks + P - 1) / P;
     if (pb < 2) pb = 2;
     pb += pb & 1;
@@ -944,6 +991,9 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
     p.ws_l = static_cast<float *>(exp_sums->data);
     p.ws_m = static_cast<float *>(max_logits->data);
     p.tmp_out = tmp_out->data;
+  } else if (generic) {
+    paged_decode_generic(generic_params(p, hd, block_size, scale), query->dtype, false, max_context_len, stream);
+    return;
   } else if (use_flat_split(S, p.Hkv * p.col_groups, max_context_len)) {
     if (query->dtype == HIPATTN_F16)
       dispatch_head_flat<half_t>(p, hd, S, max_context_len, stream);

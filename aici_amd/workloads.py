@@ -62,14 +62,14 @@ class DecodeInputs:
 
 
 def decode_inputs(seed: int, S: int, ctx_lo: int, ctx_hi: int, Hq: int, Hkv: int, d: int, dtype: torch.dtype,
-                  pool_blocks: int, device=None) -> DecodeInputs:
+                  pool_blocks: int, device=None, block_size: int = BLOCK_SIZE) -> DecodeInputs:
     """One query token per sequence; contexts uniform in [ctx_lo, ctx_hi]; block tables are
     consecutive slices of a seeded permutation of the pool (no block reused); K/V/Q ~ N(0,1).
     With `device`, the cache is filled there (seeded) instead of on the CPU."""
     g = torch.Generator().manual_seed(seed)
     rng = np.random.default_rng(seed)
     ctx = rng.integers(ctx_lo, ctx_hi + 1, size=S).astype(np.int32)
-    nblk = (ctx.astype(np.int64) + BLOCK_SIZE - 1) // BLOCK_SIZE
+    nblk = (ctx.astype(np.int64) + block_size - 1) // block_size
     assert int(nblk.sum()) <= pool_blocks, "block pool too small for the drawn contexts"
     perm = torch.randperm(pool_blocks, generator=g).numpy()
     width = int(nblk.max())
@@ -78,7 +78,7 @@ def decode_inputs(seed: int, S: int, ctx_lo: int, ctx_hi: int, Hq: int, Hkv: int
     for s in range(S):
         tables[s, :nblk[s]] = perm[pos:pos + nblk[s]]
         pos += int(nblk[s])
-    kshape, vshape = cache_shapes(pool_blocks, Hkv, d, BLOCK_SIZE, dtype)
+    kshape, vshape = cache_shapes(pool_blocks, Hkv, d, block_size, dtype)
     if device is None:
         kc = torch.randn(kshape, generator=g, dtype=torch.float32).to(dtype)
         vc = torch.randn(vshape, generator=g, dtype=torch.float32).to(dtype)

@@ -110,7 +110,12 @@ char *hipattn_mha_varlen_fwd_paged(const hipattn_tensor *q, const hipattn_tensor
  * out/query [S, Hq, d]; key_cache [nb, Hkv, d/x, BS, x]; value_cache
  * [nb, Hkv, d, BS]; block_tables int32 [S, max_blocks]; context_lens int32 [S].
  * alibi_slopes f32 [Hq] or NULL.  Runs the split-K kernel on a workspace the
- * library owns (grown with hipMalloc when a call needs more than it has). */
+ * library owns (grown with hipMalloc when a call needs more than it has).
+ * x = 16 / sizeof(dtype).  The reference's support matrix is accepted: f16,
+ * bf16 and f32; BS 8, 16 and 32; d in {64, 80, 96, 112, 128, 256}.  BS = 16 in
+ * a 2-byte type (what rLLM runs) takes the MFMA kernels; the other
+ * combinations take a plain fp32 kernel (any d <= 256 that is a multiple of
+ * x). */
 char *hipattn_paged_attention_v1(hipattn_tensor *out,
                                  const hipattn_tensor *query,
                                  const hipattn_tensor *key_cache,
@@ -127,7 +132,8 @@ char *hipattn_paged_attention_v1(hipattn_tensor *out,
  * max_logits f32 [S, Hq, P], tmp_out [S, Hq, P, d] in the cache dtype.  The
  * partition length is ceil(max_context_len / P) rounded up to a multiple of 32
  * tokens, so a caller that sizes P for the reference's 512-token partitions
- * gets 512-token partitions. */
+ * gets 512-token partitions (other block sizes and f32: a multiple of the
+ * block size, at most 8192 tokens). */
 char *hipattn_paged_attention_v2(
     hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn_tensor *max_logits,
     hipattn_tensor *tmp_out, const hipattn_tensor *query,

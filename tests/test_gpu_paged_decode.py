@@ -198,11 +198,15 @@ def test_argument_errors(device):
     c = W.decode_inputs(18, 2, 5, 40, 8, 2, 128, torch.float16, 16).to(device)
     out = torch.empty_like(c.q)
     args = (c.key_cache, c.value_cache, 2, c.scale, c.block_tables, c.context_lens)
-    with pytest.raises(HipAttnError, match="unsupported block size 32"):
-        K.paged_attention_v1(out, c.q, *args, 32, c.max_ctx)
-    with pytest.raises(HipAttnError, match="unsupported data type f32"):
+    with pytest.raises(HipAttnError, match="unsupported block size 4"):
+        K.paged_attention_v1(out, c.q, *args, 4, c.max_ctx)
+    with pytest.raises(HipAttnError, match="key_cache shape does not match"):
+        K.paged_attention_v1(out, c.q, *args, 32, c.max_ctx)        # the cache holds 16-token blocks
+    with pytest.raises(HipAttnError, match="key_cache shape does not match"):                # f32 wants x = 4
         K.paged_attention_v1(out.float(), c.q.float(), c.key_cache.float(), c.value_cache.float(), 2, c.scale,
                              c.block_tables, c.context_lens, 16, c.max_ctx)
+    with pytest.raises(HipAttnError, match="unsupported data type"):
+        K.paged_attention_v1(out.to(torch.int32), c.q.to(torch.int32), *args, 16, c.max_ctx)
     with pytest.raises(HipAttnError, match="not divisible"):
         K.paged_attention_v1(out, c.q, c.key_cache, c.value_cache, 3, c.scale, c.block_tables, c.context_lens, 16,
                              c.max_ctx)
@@ -211,3 +215,69 @@ def test_argument_errors(device):
     bad = torch.empty((2, 8, 72), dtype=torch.float16, device=c.q.device)
     with pytest.raises(HipAttnError):
         K.paged_attention_v1(bad, bad, *args, 16, c.max_ctx)
+
+
+# The rest of the reference's support matrix (attention_kernels.cu:594-700: block sizes 8/16/32,
+# float / half / bf16) runs on a plain fp32 kernel.
+FP32_TOL = 2e-5
+
+
+@pytest.mark.parametrize("case", [
+    (torch.bfloat16, 8, (32, 8, 128)), (torch.float16, 32, (32, 8, 128)), (torch.float16, 8, (32, 32, 80)),
+    (torch.bfloat16, 32, (16, 1, 96)), (torch.float32, 16, (32, 8, 128)), (torch.float32, 8, (8, 8, 64)),
+    (torch.float32, 32, (4, 4, 256)), (torch.float16, 32, (40, 2, 112)), (torch.float32, 16, (6, 3, 72)),
+])
+def test_other_block_sizes_and_fp32_match_the_oracle(device, case):
+    dtype, bs, (Hq, Hkv, d) = case
+    c = W.decode_inputs(31, 9, 1, 1500, Hq, Hkv, d, dtype, 9 * (1500 // bs + 1), block_size=bs)
+    dd = c.to(device)
+    out = torch.full_like(dd.q, float("nan"))
+    K.paged_attention_v1(out, dd.q, dd.key_cache, dd.value_cache, Hkv, c.scale, dd.block_tables, dd.context_lens, bs,
+                         c.max_ctx)
+    want = ref.paged_attention(c.q.float(), c.key_cache.float(), c.value_cache.float(), Hkv, c.scale, c.block_tables,
+                               c.context_lens, bs)
+    tol = FP32_TOL if dtype == torch.float32 else TOL[dtype]
+    assert not torch.isnan(out).any()
+    assert (out.cpu().float() - want).abs().max().item() <= tol
+    # the caller-workspace form: 3 partitions over the longest context, and far more than needed
+    for P in (3, 40):
+        out2 = torch.full_like(dd.q, float("nan"))
+        exp_sums = torch.full((9, Hq, P), float("nan"), dtype=torch.float32, device=device)
+        max_logits = torch.full_like(exp_sums, float("nan"))
+        tmp = torch.full((9, Hq, P, d), float("nan"), dtype=dtype, device=device)
+        K.paged_attention_v2(out2, exp_sums, max_logits, tmp, dd.q, dd.key_cache, dd.value_cache, Hkv, c.scale,
+                             dd.block_tables, dd.context_lens, bs, c.max_ctx)
+        assert (out2.cpu().float() - want).abs().max().item() <= tol
+
+
+@pytest.mark.parametrize("dtype,bs", [(torch.float32, 16), (torch.bfloat16, 8), (torch.float16, 32)])
+def test_other_block_sizes_edges_alibi_and_stale_slots(device, dtype, bs):
+    lens = [0, 1, bs - 1, bs, bs + 1, 255, 256, 257, 511, 512, 513, 1023, 1025]
+    S = len(lens)
+    pool = sum(lens) // bs + 2 * S
+    c = W.decode_inputs(32, S, 1, 2, 8, 2, 64, dtype, pool, block_size=bs)
+    ctx = np.array(lens, dtype=np.int32)
+    nblk = (ctx + bs - 1) // bs
+    perm = np.random.default_rng(5).permutation(pool)
+    tables = np.zeros((S, int(nblk.max())), dtype=np.int32)
+    covered = torch.zeros((pool, bs), dtype=torch.bool)
+    pos = 0
+    for s in range(S):
+        tables[s, :nblk[s]] = perm[pos:pos + nblk[s]]
+        for t in range(ctx[s]):
+            covered[tables[s, t // bs], t % bs] = True
+        pos += nblk[s]
+    c.block_tables, c.context_lens, c.max_ctx = torch.from_numpy(tables), torch.from_numpy(ctx), int(ctx.max())
+    alibi = torch.linspace(-0.3, 0.2, 8)
+    want = ref.paged_attention(c.q.float(), c.key_cache.float(), c.value_cache.float(), 2, c.scale, c.block_tables,
+                               c.context_lens, bs, alibi)
+    c.key_cache.permute(0, 3, 1, 2, 4)[~covered] = float("nan")
+    c.value_cache.permute(0, 3, 1, 2)[~covered] = float("nan")
+    dd = c.to(device)
+    out = torch.full_like(dd.q, float("nan"))
+    K.paged_attention_v1(out, dd.q, dd.key_cache, dd.value_cache, 2, c.scale, dd.block_tables, dd.context_lens, bs,
+                         c.max_ctx, alibi.to(device))
+    assert not torch.isnan(out).any()
+    assert torch.all(out[0] == 0)   # no context: a zero row, as the oracle gives
+    tol = 5e-5 if dtype == torch.float32 else TOL[dtype]
+    assert (out.cpu().float() - want).abs().max().item() <= tol
