@@ -6,8 +6,10 @@
 //  * prefill_varlen_w8_kernel (head sizes up to 128, launches of a few hundred
 //    workgroups or more): 8 wavefronts own 256 query rows, two per SIMD, each
 //    running one software-pipelined loop over 64-key tiles held in three LDS
-//    buffers, V stored transposed in LDS; a PAGED instance reads K/V from the
-//    paged cache through block tables.  Described at its definition.
+//    buffers, V stored transposed in LDS; two more instances read K/V from the
+//    paged cache through block tables -- staged through registers like the
+//    rows, or, for head sizes that fill their MFMA tiles, copied into LDS block
+//    by block with global -> LDS loads.  Described at its definition.
 //  * prefill_varlen_kernel (small launches, head sizes up to 256): a workgroup
 //    of 4 wavefronts owns 128 or 256 query rows of one (sequence, query head);
 //    each wavefront keeps QT tiles of 32 query rows, their Q operands and their
@@ -86,7 +88,7 @@ struct PrefillParams {
   // off = Lk - Lq; a negative bound is no bound (flash_attn/softmax.h:142-179, flash_api.cpp:113-120).
   // Only prefill_varlen_kernel reads these; the eight-wavefront kernel takes causal or unmasked launches.
   int win_left, win_right;
-  // K/V read straight from the paged cache (prefill_varlen_w8_kernel<..., PAGED = true>): k and v are
+  // K/V read straight from the paged cache (prefill_varlen_w8_kernel<..., W8_PAGED or W8_PAGED_DMA>): k and v are
   // the caches, position p of sequence b lives in block block_tables[b][p / 16] at offset p % 16.
   const int32_t *block_tables;
   const int32_t *context_lens;  // keys per sequence
@@ -427,6 +429,9 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
 // V^T[d][key], keys permuted so that the 8 keys a lane needs for one MFMA are
 // contiguous -- and reads both operands with ds_read_b128.
 // ---------------------------------------------------------------------------
+// Where the eight-wavefront kernel takes its K/V tiles from.
+enum { W8_ROWS = 0, W8_PAGED = 1, W8_PAGED_DMA = 2 };
+
 template <int HDP>
 struct TileW8 {
   static constexpr int KSTR = HDP + 8;   // K rows: key-major, +16 B
@@ -437,10 +442,16 @@ struct TileW8 {
   static constexpr size_t LDS_BYTES = 3 * (size_t)STAGE_ELEMS * 2;
 };
 
-template <typename T, int HDP, bool PAGED>
+template <typename T, int HDP, int MODE>
 __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams p) {
   typedef typename Vec8<T>::type vec8;
   typedef TileW8<HDP> TL;
+  constexpr bool PAGED = MODE != W8_ROWS;
+  constexpr bool DMA = MODE == W8_PAGED_DMA;
+  // W8_PAGED_DMA keeps a tile as the four block images of the cache, unpadded, in four stages.
+  constexpr int NST = DMA ? 4 : 3;
+  constexpr int STAGE_ELEMS = DMA ? 2 * BN * HDP : TL::STAGE_ELEMS;
+  constexpr int K_ELEMS = DMA ? BN * HDP : TL::K_ELEMS;
   constexpr int KSTEPS = HDP / 16;
   constexpr int NDT = HDP / 32;
   constexpr int CPR = HDP / 8;                // 16-byte chunks per K row
@@ -496,13 +507,13 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   // 16 bytes per row, 4 rows per instruction) and turned through a private piece of LDS buffers 1 and 2,
   // which no tile reaches before the first barrier.
   constexpr int QSTR = HDP + 8;  // row pitch of the turned Q tile, elements
-  constexpr bool Q_VIA_LDS = (size_t)8 * 32 * QSTR <= (size_t)2 * TL::STAGE_ELEMS;
+  constexpr bool Q_VIA_LDS = (size_t)8 * 32 * QSTR <= (size_t)(NST - 1) * STAGE_ELEMS;
   vec8 qreg[KSTEPS];
   auto load_q = [&]() {
     if constexpr (Q_VIA_LDS) {
       constexpr int CPRQ = HDP / 8;
       constexpr int NQL = (32 * CPRQ + 63) / 64;
-      T *qst = smem + TL::STAGE_ELEMS + wave * (32 * QSTR);
+      T *qst = smem + STAGE_ELEMS + wave * (32 * QSTR);
       u32x4_t raw[NQL];
 #pragma unroll
       for (int it = 0; it < NQL; it++) {
@@ -572,34 +583,111 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   u32x4_t vstp[PAGED ? NLOADVP : 1];
   int staged_k0 = 0;  // first key of the tile held in the staging registers
   const int32_t *table_row = PAGED ? p.block_tables + (int64_t)b * p.table_stride : nullptr;
-  auto table_block = [&](int col) -> int64_t {
-    const int64_t blk = table_row[min(col, p.table_cols - 1)];
-    return blk < 0 ? 0 : (blk >= p.num_blocks ? p.num_blocks - 1 : blk);
+  // The block ids of 64 table columns (16 tiles) sit one per lane (columns past the context repeat its
+  // last one), and a tile's four ids are lane reads into scalar registers: no tile waits for a table
+  // read.  The next group is asked for one tile before it is needed and the ids are clamped to the cache
+  // where they are used, so that nothing waits for the read where it is issued.
+  int tbl_cur = 0, tbl_nxt = 0;
+  auto load_ids = [&](int group) -> int {
+    const int last_col = min((Lk - 1) >> 4, p.table_cols - 1);
+    return table_row[max(min(group * 64 + lane, last_col), 0)];
   };
+  auto block_id = [&](int idx) -> int64_t {
+    const int blk = __builtin_amdgcn_readlane(tbl_cur, idx);
+    return blk < 0 ? 0 : (blk >= p.num_blocks ? p.num_blocks - 1 : (int64_t)blk);
+  };
+  // After a tile's ids are read: the last but one tile of a group asks for the next group's ids, the last
+  // one switches to them.
+  auto next_ids = [&](int tile) {
+    if ((tile & 15) == 14) tbl_nxt = load_ids((tile >> 4) + 1);
+    if ((tile & 15) == 15) tbl_cur = tbl_nxt;
+  };
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   auto load_tile_paged = [&](int tile) {
     const int k0 = tile * BN;
     staged_k0 = k0;
-    // Blocks wholly or partly inside the context; a block past it re-reads the last one (its keys are
-    // masked, its V runs cleared before they reach LDS).
-    const int last_col = (Lk - 1) >> 4;
-    int64_t blk[4];
-#pragma unroll
-    for (int r = 0; r < 4; r++) blk[r] = table_block(min(k0 / 16 + r, last_col));
+    const int slot = tile & 15;
+    // A wavefront's 64 runs lie in one block (a block has 2 HDP runs of K and of V), so the block's
+    // address is scalar and the lane adds its run.  Blocks past the context re-read the last one
+    // (their keys are masked, their V runs cleared before they reach LDS).
 #pragma unroll
     for (int i = 0; i < NLOADK; i++) {
-      const int u = min(tid + 512 * i, K_CHUNKS - 1);
-      const int r = u / K_PER_BLOCK, rem = u % K_PER_BLOCK;
+      const int ub = min(wave_u * 64 + 512 * i, K_CHUNKS - 64);
+      const int r = ub / K_PER_BLOCK, rem = ub % K_PER_BLOCK + lane;
       const int c8 = min(rem / 16, d_chunks - 1), tok = rem % 16;
-      const int64_t bs = r == 0 ? blk[0] : (r == 1 ? blk[1] : (r == 2 ? blk[2] : blk[3]));
-      kst[i] = *reinterpret_cast<const u32x4_t *>(kp + bs * p.kc_block + (c8 * 16 + tok) * 8);
+      const int64_t bs = block_id(slot * 4 + r);
+      const char *base = reinterpret_cast<const char *>(kp + bs * p.kc_block);
+      kst[i] = *reinterpret_cast<const u32x4_t *>(base + (uint32_t)((c8 * 16 + tok) * 8 * (int)sizeof(T)));
     }
 #pragma unroll
     for (int i = 0; i < NLOADVP; i++) {
-      const int u = min(tid + 512 * i, 4 * V_PER_BLOCK - 1);
-      const int r = u / V_PER_BLOCK, rem = u % V_PER_BLOCK;
+      const int ub = min(wave_u * 64 + 512 * i, 4 * V_PER_BLOCK - 64);
+      const int r = ub / V_PER_BLOCK, rem = ub % V_PER_BLOCK + lane;
       const int drow = min(rem / 2, p.d - 1), half = rem % 2;
-      const int64_t bs = r == 0 ? blk[0] : (r == 1 ? blk[1] : (r == 2 ? blk[2] : blk[3]));
-      vstp[i] = *reinterpret_cast<const u32x4_t *>(vp + bs * p.vc_block + drow * 16 + half * 8);
+      const int64_t bs = block_id(slot * 4 + r);
+      const char *base = reinterpret_cast<const char *>(vp + bs * p.vc_block);
+      vstp[i] = *reinterpret_cast<const u32x4_t *>(base + (uint32_t)((drow * 16 + half * 8) * (int)sizeof(T)));
+    }
+    next_ids(tile);
+  };
+  // W8_PAGED_DMA (d == HDP): the tile's blocks go from the cache into LDS as they are, 1 KiB per
+  // instruction (lane l's 16 bytes land at M0 + 16 l), no staging registers and no LDS writes.  A block of
+  // one kv head is HDP * 32 contiguous bytes of K and as many of V; the tile's 8 * PIECES pieces are dealt
+  // round-robin to the 8 wavefronts.  K pieces keep the cache's order; in a V piece (32 rows x 16 tokens)
+  // lane l fetches tokens 8 (l / 32) .. + 8 of row l % 32.
+  constexpr int BLK_ELEMS = HDP * 16;
+  constexpr int PIECES = HDP / 32;  // 1 KiB pieces per block image
+  constexpr int NDMA = HDP / 32;    // instructions per wavefront and tile
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem_raw;
+  const unsigned dma_k_lane = lane * 16, dma_v_lane = c * 32 + g * 16;
+  auto dma_piece = [&](int tile, int i) {
+    const int slot = tile & 15;
+    const unsigned stage = lds0 + (unsigned)((tile % NST) * STAGE_ELEMS * (int)sizeof(T));
+    const int q = wave_u + 8 * i;
+    const bool is_v = q >= 4 * PIECES;
+    const int qq = is_v ? q - 4 * PIECES : q;
+    const int r = qq / PIECES, n = qq % PIECES;
+    const int64_t bs = block_id(slot * 4 + r);
+    const char *src = reinterpret_cast<const char *>(is_v ? vp + bs * p.vc_block : kp + bs * p.kc_block) + n * 1024;
+    const unsigned dst = stage + (unsigned)(((is_v ? K_ELEMS : 0) + r * BLK_ELEMS + n * 512) * (int)sizeof(T));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(dst), "v"(is_v ? dma_v_lane : dma_k_lane), "s"(src)
+                 : "memory");
+    if (i == NDMA - 1) next_ids(tile);
+  };
+  auto dma_tile = [&](int tile) {
+#pragma unroll
+    for (int i = 0; i < NDMA; i++) dma_piece(tile, i);
+  };
+  // Waits until this wavefront's pieces of `tile` have landed (`newer`: the pieces of the tile after it
+  // were issued later and may still fly), then clears the V tokens past the context in them: stale
+  // cache contents may be NaN, which a zero probability would not neutralise.
+  auto dma_wait = [&](int tile, bool newer) {
+    if (newer)
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (tile * BN + BN > Lk) {
+      T *vs = smem + (tile % NST) * STAGE_ELEMS + K_ELEMS;
+#pragma unroll
+      for (int i = 0; i < NDMA; i++) {
+        const int q = wave_u + 8 * i;
+        if (q >= 4 * PIECES) {
+          const int r = (q - 4 * PIECES) / PIECES, n = (q - 4 * PIECES) % PIECES;
+          const int alive = Lk - (tile * BN + r * 16 + g * 8);  // tokens of this lane's run inside the context
+          if (alive < 8) {
+            u32x4_t *run = reinterpret_cast<u32x4_t *>(vs + r * BLK_ELEMS + n * 512 + lane * 8);
+            u32x4_t o = *run;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+              const int a2 = alive - 2 * w;
+              o[w] &= a2 <= 0 ? 0u : (a2 == 1 ? 0xffffu : 0xffffffffu);
+            }
+            *run = o;
+          }
+        }
+      }
     }
   };
   auto load_tile_rows = [&](int tile) {
@@ -633,8 +721,8 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       load_tile_rows(tile);
   };
   auto store_tile_paged = [&](int stage) {
-    T *ks = smem + stage * TL::STAGE_ELEMS;
-    T *vs = ks + TL::K_ELEMS;
+    T *ks = smem + stage * STAGE_ELEMS;
+    T *vs = ks + K_ELEMS;
 #pragma unroll
     for (int i = 0; i < NLOADK; i++) {
       const int u = tid + 512 * i;
@@ -669,8 +757,8 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     }
   };
   auto store_tile_rows = [&](int stage) {
-    T *ks = smem + stage * TL::STAGE_ELEMS;
-    T *vs = ks + TL::K_ELEMS;
+    T *ks = smem + stage * STAGE_ELEMS;
+    T *vs = ks + K_ELEMS;
 #pragma unroll
     for (int i = 0; i < NLOADK; i++) {
       const int idx = tid + 512 * i;
@@ -706,24 +794,45 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       store_tile_rows(stage);
   };
 
-  if (n_tiles > 0) load_tile(0);
-  load_q();
-  if (n_tiles > 0) {
-    store_tile(0);
-    if (n_tiles > 1) load_tile(1);
+  if (PAGED && n_tiles > 0) tbl_cur = load_ids(0);
+  if constexpr (DMA) {
+    // Tile 0 flies into stage 0 while Q is turned through stages 1..3; tiles 1 and 2 follow once every
+    // wavefront has its Q.
+    if (n_tiles > 0) dma_tile(0);
+    load_q();
+    if (n_tiles > 0) dma_wait(0, false);
+    __syncthreads();
+    if (n_tiles > 1) dma_tile(1);
+    if (n_tiles > 2) dma_tile(2);
+  } else {
+    if (n_tiles > 0) load_tile(0);
+    load_q();
+    if (n_tiles > 0) {
+      store_tile(0);
+      if (n_tiles > 1) load_tile(1);
+    }
+    __syncthreads();
   }
-  __syncthreads();
 
-  const int k_lane_off = c * TL::KSTR + g * 8;
-  const int v_lane_off = c * TL::VTSTR + g * 8;
+  // Operand reads.  Staged tiles: K rows and V^T rows with 16 bytes of padding.  Block images: lane c is
+  // MFMA row m = [a1 a0 g' b1 b0] and reads token [g' a0 b1 b0] of block a1 of its 32-key half, so that the
+  // 8 scores a lane holds for one P.V step belong to 8 consecutive tokens of one block -- the order in which
+  // a V row lies in the cache.  Sixteen consecutive lanes then read one whole 256-byte run [chunk][16
+  // tokens] of K, and the 32 lanes of a half-wavefront 512 consecutive bytes of V (the DMA places the two
+  // 8-token halves of 32 rows one after the other): no padding is needed.
+  const int k_lane_off = DMA ? (c >> 4) * (HDP * 16) + g * 128 + (((c >> 2) & 1) * 8 + ((c >> 3) & 1) * 4 + (c & 3)) * 8
+                             : c * TL::KSTR + g * 8;
+  const int v_lane_off = DMA ? g * 256 + c * 8 : c * TL::VTSTR + g * 8;
+  constexpr int K_HALF = DMA ? 2 * HDP * 16 : 32 * TL::KSTR;  // elements between the two 32-key halves of a K tile
+  constexpr int K_STEP = DMA ? 256 : 16;                      // ... between contraction steps (16 head elements)
   const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // S^T = K . Q^T of one tile on its own (used for tile 0): both 32-key halves,
   // LDS reads two contraction steps ahead of the MFMAs that consume them.
   auto phase_qk = [&](int buf, f32x16_t(&s)[2]) {
-    const T *ks_base = smem + buf * TL::STAGE_ELEMS;
+    const T *ks_base = smem + buf * STAGE_ELEMS;
     auto rd = [&](int kt, int ks) -> vec8 {
-      return *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + kt * 32 * TL::KSTR + ks * 16);
+      return *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + kt * K_HALF + ks * K_STEP);
     };
     vec8 ka[3][2];
     ka[0][0] = rd(0, 0);
@@ -763,9 +872,9 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   auto qk_softmax = [&](auto do_qk, int j, f32x16_t(&s)[2], f32x16_t(&sn)[2], vec8(&pk)[2][2]) {
     constexpr bool DO_QK = decltype(do_qk)::value;
     const int k0 = j * BN;
-    const T *ks_base = smem + ((j + 1) % 3) * TL::STAGE_ELEMS;
+    const T *ks_base = smem + ((j + 1) % NST) * STAGE_ELEMS;
     auto rd = [&](int n) -> vec8 {
-      return *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + (n & 1) * 32 * TL::KSTR + (n >> 1) * 16);
+      return *reinterpret_cast<const vec8 *>(ks_base + k_lane_off + (n & 1) * K_HALF + (n >> 1) * K_STEP);
     };
     vec8 ka[QK_DEPTH + 1];
     if (DO_QK) {
@@ -790,7 +899,8 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       for (int kt = 0; kt < 2; kt++)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-          const int key = k0 + kt * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
+          const int key = DMA ? k0 + kt * 32 + ((i >> 3) & 1) * 16 + g * 8 + ((i >> 2) & 1) * 4 + (i & 3)
+                              : k0 + kt * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
           if (key > limit) s[kt][i] = -INFINITY;
         }
     }
@@ -833,11 +943,12 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   // P(j).V(j) with the staging for later tiles in its shadow.
   constexpr int PV_STEPS = NDT * 4;
   auto pv_stage = [&](bool live, int j, vec8(&pk)[2][2]) {
-    const T *vs_base = smem + (j % 3) * TL::STAGE_ELEMS + TL::K_ELEMS;
+    const T *vs_base = smem + (j % NST) * STAGE_ELEMS + K_ELEMS;
     // Step n = (contraction step n / NDT, output tile n % NDT): consecutive MFMAs go to different
     // accumulators, so none waits for the result of the one before it.
     auto rd = [&](int n) -> vec8 {
       const int dt = n % NDT, ks = n / NDT, kt = ks / 2, half = ks % 2;
+      if constexpr (DMA) return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + ks * (HDP * 16) + dt * 512);
       return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + dt * 32 * TL::VTSTR + kt * 32 + half * 16);
     };
     if (live) {
@@ -850,12 +961,23 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         __builtin_amdgcn_sched_barrier(0);
         acc[n % NDT] = Mfma32<T>::run(va[n % 4], pk[(n / NDT) / 2][(n / NDT) % 2], acc[n % NDT]);
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (DMA) {
+          // one piece every few MFMAs: issued back to back they queue up in front of the memory pipeline
+          if (n % (PV_STEPS / NDMA) == 1 && j + 3 < n_tiles) {
+            dma_piece(j + 3, n / (PV_STEPS / NDMA));
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
         if (n == 1) {
-          if (j + 2 < n_tiles) store_tile((j + 2) % 3);
-          if (j + 3 < n_tiles) load_tile(j + 3);
+          if constexpr (!DMA) {
+            if (j + 2 < n_tiles) store_tile((j + 2) % 3);
+            if (j + 3 < n_tiles) load_tile(j + 3);
+          }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+    } else if constexpr (DMA) {
+      if (j + 3 < n_tiles) dma_tile(j + 3);
     } else {
       if (j + 2 < n_tiles) store_tile((j + 2) % 3);
       if (j + 3 < n_tiles) load_tile(j + 3);
@@ -865,8 +987,12 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   f32x16_t s_a[2], s_b[2];
   // S(0) has nothing to hide behind; tile 1 is staged while it runs.
   if (n_tiles > 0 && !skip_tile(0)) phase_qk(0, s_a);
-  if (n_tiles > 1) store_tile(1);
-  if (n_tiles > 2) load_tile(2);
+  if constexpr (DMA) {
+    if (n_tiles > 1) dma_wait(1, n_tiles > 2);
+  } else {
+    if (n_tiles > 1) store_tile(1);
+    if (n_tiles > 2) load_tile(2);
+  }
   lds_barrier();
 
   auto iteration = [&](int j, f32x16_t(&s)[2], f32x16_t(&sn)[2]) {
@@ -883,6 +1009,9 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     PHASE_STAMP(1);
     pv_stage(live, j, pk);
     PHASE_STAMP(2);
+    if constexpr (DMA) {
+      if (j + 2 < n_tiles) dma_wait(j + 2, j + 3 < n_tiles);
+    }
     lds_barrier();
     PHASE_STAMP(3);
   };
@@ -934,19 +1063,20 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   }
 }
 
-template <typename T, int HDP, bool PAGED = false>
+template <typename T, int HDP, int MODE = W8_ROWS>
 void launch_prefill_w8(PrefillParams p, hipStream_t stream) {
   static bool attr_set = false;  // benign race: setting twice is harmless
-  auto kernel = prefill_varlen_w8_kernel<T, HDP, PAGED>;
+  auto kernel = prefill_varlen_w8_kernel<T, HDP, MODE>;
+  constexpr size_t lds_bytes = MODE == W8_PAGED_DMA ? (size_t)4 * 2 * BN * HDP * 2 : TileW8<HDP>::LDS_BYTES;
   if (!attr_set) {
     HA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)TileW8<HDP>::LDS_BYTES));
+                               (int)lds_bytes));
     attr_set = true;
   }
   p.n_qblocks = (p.max_q + 255) / 256;
   const int64_t n_wg = (int64_t)p.n_qblocks * p.batch * p.Hq;
   HA_CHECK(n_wg <= 0x7fffffff, "mha_varlen_fwd: too many workgroups");
-  kernel<<<dim3((unsigned)n_wg), 512, TileW8<HDP>::LDS_BYTES, stream>>>(p);
+  kernel<<<dim3((unsigned)n_wg), 512, lds_bytes, stream>>>(p);
   check_launch("mha_varlen_fwd");
 }
 
@@ -1130,13 +1260,21 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
 template <typename T>
 void dispatch_paged(const PrefillParams &p, hipStream_t stream) {
   const int hdp = ((p.d + 31) / 32) * 32;
+  // Head sizes that fill their MFMA tiles take the block images as they are; the others are staged
+  // through registers, which pads them.  HIPATTN_PAGED_PREFILL_DMA=0 forces the staged form (tuning aid).
+  const char *force = getenv("HIPATTN_PAGED_PREFILL_DMA");
+  const bool dma = p.d == hdp && !(force && force[0] == '0');
+#define HA_W8P(H)                                              \
+  if (dma) launch_prefill_w8<T, H, W8_PAGED_DMA>(p, stream);   \
+  else launch_prefill_w8<T, H, W8_PAGED>(p, stream)
   switch (hdp) {
-    case 32: launch_prefill_w8<T, 32, true>(p, stream); break;
-    case 64: launch_prefill_w8<T, 64, true>(p, stream); break;
-    case 96: launch_prefill_w8<T, 96, true>(p, stream); break;
-    case 128: launch_prefill_w8<T, 128, true>(p, stream); break;
+    case 32: HA_W8P(32); break;
+    case 64: HA_W8P(64); break;
+    case 96: HA_W8P(96); break;
+    case 128: HA_W8P(128); break;
     default: fail("mha_varlen_fwd_paged: head size %d not supported (at most 128)", p.d);
   }
+#undef HA_W8P
 }
 
 void mha_varlen_fwd_paged_impl(const hipattn_tensor *q, const hipattn_tensor *key_cache,

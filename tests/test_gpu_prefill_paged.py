@@ -17,6 +17,18 @@ from tests.common import TOL, make_cache
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["auto", "staged"])
+def tile_route(request, monkeypatch):
+    """Head sizes that fill their MFMA tiles (32, 64, 96, 128) have their tiles copied from the cache into
+    LDS as block images; the others -- and every size when HIPATTN_PAGED_PREFILL_DMA=0 -- are staged
+    through registers.  Every test runs both ways."""
+    if request.param == "auto":
+        monkeypatch.delenv("HIPATTN_PAGED_PREFILL_DMA", raising=False)
+    else:
+        monkeypatch.setenv("HIPATTN_PAGED_PREFILL_DMA", "0")
+    return request.param
+
+
 def paged_case(seed, seqs, Hq, Hkv, d, dtype, pool):
     """seqs: (prior, new) token counts.  Every context's K/V (prior and new) is in the cache; every slot no
     context covers holds NaN, as an uninitialised cache may."""
