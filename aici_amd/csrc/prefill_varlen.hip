@@ -632,29 +632,46 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   };
   // W8_PAGED_DMA (d == HDP): the tile's blocks go from the cache into LDS as they are, 1 KiB per
   // instruction (lane l's 16 bytes land at M0 + 16 l), no staging registers and no LDS writes.  A block of
-  // one kv head is HDP * 32 contiguous bytes of K and as many of V; the tile's 8 * PIECES pieces are dealt
-  // round-robin to the 8 wavefronts.  K pieces keep the cache's order; in a V piece (32 rows x 16 tokens)
-  // lane l fetches tokens 8 (l / 32) .. + 8 of row l % 32.
+  // one kv head is HDP * 32 contiguous bytes of K and as many of V.  Wavefront w copies one such image per
+  // tile: K (w even) or V (w odd) of block w / 2, as HDP / 32 pieces.  K pieces keep the cache's order; in
+  // a V piece (32 rows x 16 tokens) lane l fetches tokens 8 (l / 32) .. + 8 of row l % 32.  What sits one
+  // per lane here is the byte offset of the block in this wavefront's cache, so that a tile costs two lane
+  // reads and an add.
   constexpr int BLK_ELEMS = HDP * 16;
-  constexpr int PIECES = HDP / 32;  // 1 KiB pieces per block image
-  constexpr int NDMA = HDP / 32;    // instructions per wavefront and tile
+  constexpr int NDMA = HDP / 32;  // instructions per wavefront and tile
   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem_raw;
-  const unsigned dma_k_lane = lane * 16, dma_v_lane = c * 32 + g * 16;
+  const int dma_v = wave_u & 1, dma_r = wave_u >> 1;
+  const unsigned dma_lane = dma_v ? c * 32 + g * 16 : lane * 16;
+  const char *dma_base = reinterpret_cast<const char *>(dma_v ? vp : kp);
+  const int64_t dma_blk_bytes = (dma_v ? p.vc_block : p.kc_block) * (int64_t)sizeof(T);
+  int64_t tbl_off = 0;
+  auto ids_to_offsets = [&](int blk) -> int64_t {
+    const int64_t bid = blk < 0 ? 0 : (blk >= p.num_blocks ? p.num_blocks - 1 : (int64_t)blk);
+    return bid * dma_blk_bytes;
+  };
   auto dma_piece = [&](int tile, int i) {
-    const int slot = tile & 15;
-    const unsigned stage = lds0 + (unsigned)((tile % NST) * STAGE_ELEMS * (int)sizeof(T));
-    const int q = wave_u + 8 * i;
-    const bool is_v = q >= 4 * PIECES;
-    const int qq = is_v ? q - 4 * PIECES : q;
-    const int r = qq / PIECES, n = qq % PIECES;
-    const int64_t bs = block_id(slot * 4 + r);
-    const char *src = reinterpret_cast<const char *>(is_v ? vp + bs * p.vc_block : kp + bs * p.kc_block) + n * 1024;
-    const unsigned dst = stage + (unsigned)(((is_v ? K_ELEMS : 0) + r * BLK_ELEMS + n * 512) * (int)sizeof(T));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(dst), "v"(is_v ? dma_v_lane : dma_k_lane), "s"(src)
-                 : "memory");
-    if (i == NDMA - 1) next_ids(tile);
+    const int idx = (tile & 15) * 4 + dma_r;
+    const unsigned lo = __builtin_amdgcn_readlane((int)(uint32_t)tbl_off, idx);
+    const unsigned hi = __builtin_amdgcn_readlane((int)(uint32_t)(tbl_off >> 32), idx);
+    const char *src = dma_base + (((uint64_t)hi << 32) | lo);
+    // the instruction's offset field moves both ends of the copy: the address in memory and the one in LDS
+    const unsigned dst = lds0 + (unsigned)(((tile % NST) * STAGE_ELEMS + dma_v * K_ELEMS + dma_r * BLK_ELEMS) * (int)sizeof(T));
+#define HA_DMA_PIECE(OFF)                                                                          \
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:" #OFF \
+               :                                                                                   \
+               : "s"(dst), "v"(dma_lane), "s"(src)                                                 \
+               : "memory")
+    switch (i) {
+      case 0: HA_DMA_PIECE(0); break;
+      case 1: HA_DMA_PIECE(1024); break;
+      case 2: HA_DMA_PIECE(2048); break;
+      default: HA_DMA_PIECE(3072); break;
+    }
+#undef HA_DMA_PIECE
+    if (i == NDMA - 1) {
+      if ((tile & 15) == 14) tbl_nxt = load_ids((tile >> 4) + 1);
+      if ((tile & 15) == 15) tbl_off = ids_to_offsets(tbl_nxt);
+    }
   };
   auto dma_tile = [&](int tile) {
 #pragma unroll
@@ -668,24 +685,20 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
     else
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (tile * BN + BN > Lk) {
-      T *vs = smem + (tile % NST) * STAGE_ELEMS + K_ELEMS;
+    if (dma_v && tile * BN + BN > Lk) {
+      T *vs = smem + (tile % NST) * STAGE_ELEMS + K_ELEMS + dma_r * BLK_ELEMS;
+      const int alive = Lk - (tile * BN + dma_r * 16 + g * 8);  // tokens of this lane's runs inside the context
+      if (alive < 8) {
 #pragma unroll
-      for (int i = 0; i < NDMA; i++) {
-        const int q = wave_u + 8 * i;
-        if (q >= 4 * PIECES) {
-          const int r = (q - 4 * PIECES) / PIECES, n = (q - 4 * PIECES) % PIECES;
-          const int alive = Lk - (tile * BN + r * 16 + g * 8);  // tokens of this lane's run inside the context
-          if (alive < 8) {
-            u32x4_t *run = reinterpret_cast<u32x4_t *>(vs + r * BLK_ELEMS + n * 512 + lane * 8);
-            u32x4_t o = *run;
+        for (int i = 0; i < NDMA; i++) {
+          u32x4_t *run = reinterpret_cast<u32x4_t *>(vs + i * 512 + lane * 8);
+          u32x4_t o = *run;
 #pragma unroll
-            for (int w = 0; w < 4; w++) {
-              const int a2 = alive - 2 * w;
-              o[w] &= a2 <= 0 ? 0u : (a2 == 1 ? 0xffffu : 0xffffffffu);
-            }
-            *run = o;
+          for (int w = 0; w < 4; w++) {
+            const int a2 = alive - 2 * w;
+            o[w] &= a2 <= 0 ? 0u : (a2 == 1 ? 0xffffu : 0xffffffffu);
           }
+          *run = o;
         }
       }
     }
@@ -796,6 +809,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
 
   if (PAGED && n_tiles > 0) tbl_cur = load_ids(0);
   if constexpr (DMA) {
+    tbl_off = ids_to_offsets(tbl_cur);
     // Tile 0 flies into stage 0 while Q is turned through stages 1..3; tiles 1 and 2 follow once every
     // wavefront has its Q.
     if (n_tiles > 0) dma_tile(0);
