@@ -308,6 +308,7 @@ def main() -> None:
 
     from aici_amd import kernels as K
     from aici_amd import workloads as W
+    from aici_amd import paged
 
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
@@ -410,7 +411,34 @@ def main() -> None:
                          "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
                          "kernel": "prefill_varlen_w8_kernel, HIP events on the launch stream"},
         }
-        del p
+        # The same rows with K/V read from the paged cache they were scattered into (what an engine step
+        # has at hand: rLLM writes the cache first, llm/mod.rs:147-164, and gathers back from it).
+        nb = sum((l + 15) // 16 for l in p.lens_k)
+        perm = torch.randperm(nb + 64, generator=torch.Generator().manual_seed(3)).tolist()
+        tables = torch.zeros((len(p.lens_k), max((l + 15) // 16 for l in p.lens_k)), dtype=torch.int32)
+        slots, pos = [], 0
+        for i, l in enumerate(p.lens_k):
+            n = (l + 15) // 16
+            tables[i, :n] = torch.tensor(perm[pos:pos + n], dtype=torch.int32)
+            slots += W.slots_for(perm[pos:pos + n], l)
+            pos += n
+        kc, vc = paged.alloc_gpu_cache_layer(nb + 64, p.k.shape[1], p.k.shape[2], 16, p.k.dtype, dev)
+        K.reshape_and_cache(p.k, p.v, kc, vc, torch.tensor(slots, dtype=torch.int64, device=dev))
+        tb, ctx = tables.to(dev), torch.tensor(p.lens_k, dtype=torch.int32, device=dev)
+
+        def paged_step():
+            K.flash_attn_varlen_paged(p.q, kc, vc, tb, p.cu_q, ctx, p.max_q, p.max_k, p.scale, True)
+
+        for _ in range(10):
+            paged_step()
+        torch.cuda.synchronize()
+        ql = event_times_ms(paged_step, psteps, stream)
+        qms = sum(ql) / len(ql)
+        line["prefill"]["from_paged_cache"] = {
+            "value": round(p.flops() / (qms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": round(qms, 4),
+            "frac": round(p.flops() / (qms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "kernel": "prefill_varlen_w8_kernel, block images copied global -> LDS (hipattn_mha_varlen_fwd_paged)"}
+        del p, kc, vc
 
     # ---- optional: the streaming helpers -------------------------------------------------------------
     if args.streaming:
