@@ -471,11 +471,15 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   const int g = lane >> 5;
   const int c = lane & 31;
 
+  // Workgroups in launch order: query head fastest (the heads of a kv group land on one XCD and share its
+  // L2), then the row blocks of a sequence, last rows -- the longest stretch of keys under the causal mask --
+  // first, then the sequence: a sequence's row blocks run at the same time and find its keys in L2 (against
+  // sequence-fastest order: -1.5 % on 8 x 4096 self-attention, -2.8 % on 512-row chunks over 8192 cached keys).
   int id = blockIdx.x;
   const int slot = id % p.Hq;
   id /= p.Hq;
-  const int b = id % p.batch;
-  const int qb = p.n_qblocks - 1 - id / p.batch;
+  const int b = id / p.n_qblocks;
+  const int qb = p.n_qblocks - 1 - id % p.n_qblocks;
   const int h = (slot % p.Hkv) * p.G + slot / p.Hkv;
   const int kvh = h / p.G;
 
