@@ -77,7 +77,8 @@ SEQS = [(0, 5), (0, 64), (100, 33), (1000, 256), (17, 1), (0, 300), (63, 65), (2
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("heads", [(32, 8, 128), (32, 32, 80), (8, 2, 64), (4, 4, 32), (6, 1, 96)])
+@pytest.mark.parametrize("heads", [(32, 8, 128), (32, 32, 80), (8, 2, 64), (4, 4, 32), (6, 1, 96), (8, 2, 112), (4, 4, 120),
+                                   (4, 2, 8)])
 def test_matches_oracle(device, dtype, heads):
     Hq, Hkv, d = heads
     c = paged_case(31, SEQS, Hq, Hkv, d, dtype, 420)
