@@ -84,6 +84,7 @@ _ERR_FUNCS = {
     "hipattn_copy_blocks_2": [TP, TP, TP, TP, c_void_p],
     "hipattn_swap_blocks": [TP, c_int, TP, c_int, POINTER(c_int64), c_int64, c_void_p],
     "hipattn_rotary_embedding": [TP, TP, TP, c_int, TP, c_bool, c_void_p],
+    "hipattn_rotary_embedding_and_cache": [TP, TP, TP, TP, c_int, TP, c_bool, TP, TP, TP, c_void_p],
     "hipattn_rms_norm": [TP, TP, TP, c_float, c_void_p],
     "hipattn_fused_add_rms_norm": [TP, TP, TP, c_float, c_void_p],
     "hipattn_silu_and_mul": [TP, TP, c_void_p],

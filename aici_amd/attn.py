@@ -34,6 +34,13 @@ class RotaryEmbedding:
         idx_theta = torch.arange(max_len, dtype=torch.float32).reshape(max_len, 1).matmul(theta.reshape(1, -1))
         return torch.cat([idx_theta.cos().to(dtype), idx_theta.sin().to(dtype)], dim=-1).contiguous()
 
+    def forward_and_cache(self, positions: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                          key_cache: torch.Tensor, value_cache: torch.Tensor, slot_mapping: torch.Tensor) -> None:
+        """forward() and the scatter of the rotated keys and of v [T, Hkv, d] into the cache, in one launch;
+        q [T, Hq*d] and k [T, Hkv*d] (row strides allowed) are rotated in place."""
+        kernels.rotary_embedding_and_cache(positions, q, k, v, self.head_dim, self.cos_sin, True, key_cache,
+                                           value_cache, slot_mapping)
+
     def forward(self, positions: torch.Tensor, q: torch.Tensor, k: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         q = q.reshape(-1, self.num_attention_heads * self.head_dim)
         k = k.reshape(-1, self.num_key_value_heads * self.head_dim)
@@ -59,8 +66,9 @@ class RmsNorm:
 
 def varlen_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch_info: BatchInfo, key_cache: torch.Tensor,
                 value_cache: torch.Tensor, softmax_scale: Optional[float] = None,
-                paged_prefill: bool = False) -> torch.Tensor:
-    """mod.rs:318-354: q [T,Hq,d], k/v [T,Hkv,d] -> [T, Hq*d].
+                paged_prefill: bool = False, cached: bool = False) -> torch.Tensor:
+    """mod.rs:318-354: q [T,Hq,d], k/v [T,Hkv,d] -> [T, Hq*d].  `cached`: the new K/V are in the cache
+    already (kernels.rotary_embedding_and_cache) and the scatter is skipped.
 
     batch_info must already live on the GPU.  The whole composition (scatter,
     gather, varlen prefill rows, paged decode rows) is one C-ABI call.  With
@@ -77,7 +85,7 @@ def varlen_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch_info: B
             raise ValueError("paged_prefill needs batch_info.multi_block_tables (slots must follow the blocks in order)")
         has_m, has_p = batch_info.q_multi > 0, batch_info.q_multi < T
         call("hipattn_varlen_attn_paged", _desc(q, "q"), _desc(k, "k"), _desc(v, "v"), _desc(key_cache, "key_cache"),
-             _desc(value_cache, "value_cache"), _desc(batch_info.slot_mapping, "slot_mapping"),
+             _desc(value_cache, "value_cache"), None if cached else _desc(batch_info.slot_mapping, "slot_mapping"),
              _desc(batch_info.multi_block_tables, "multi_block_tables") if has_m else None,
              _desc(batch_info.seqlens_q, "seqlens_q") if has_m else None,
              _desc(batch_info.multi_context_lens, "multi_context_lens") if has_m else None, int(batch_info.q_multi),
@@ -93,7 +101,7 @@ def varlen_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch_info: B
     has_multi = batch_info.q_multi > 0
     has_paged = batch_info.q_multi < T
     call("hipattn_varlen_attn", _desc(q, "q"), _desc(k, "k"), _desc(v, "v"), _desc(key_cache, "key_cache"),
-         _desc(value_cache, "value_cache"), _desc(batch_info.slot_mapping, "slot_mapping"),
+         _desc(value_cache, "value_cache"), None if cached else _desc(batch_info.slot_mapping, "slot_mapping"),
          _desc(batch_info.gather_mapping, "gather_mapping") if has_multi else None,
          _desc(batch_info.seqlens_q, "seqlens_q") if has_multi else None,
          _desc(batch_info.seqlens_k, "seqlens_k") if has_multi else None, int(batch_info.q_multi),

@@ -396,6 +396,86 @@ __global__ __launch_bounds__(256) void cache_move_scalar_kernel(
   }
 }
 
+// rotary_embedding followed by reshape_and_cache for the new tokens of a step, in one launch (a decode step
+// is bound by its launches, not by these few kilobytes): a workgroup per token rotates the query heads in
+// place, rotates the key heads in place and writes them to the cache from the same registers, and
+// scatters the value heads.  NeoX layout, 2-byte types, 16-byte steps; arithmetic and rounding are those of
+// rotary_neox_vec8_kernel, so the results equal the two calls bit for bit.  A position outside the table
+// leaves its row unrotated (it is still cached); a negative slot or one past the cache is not cached.
+template <typename T, typename Pos, typename Slot>
+__global__ __launch_bounds__(256) void rotary_cache_kernel(const Pos *__restrict__ positions, T *__restrict__ query,
+                                                           T *__restrict__ key, const T *__restrict__ value,
+                                                           const T *__restrict__ cos_sin, int rot_dim, int64_t max_pos,
+                                                           int64_t q_stride, int64_t k_stride, int64_t v_tok_stride,
+                                                           int64_t v_head_stride, int num_q_heads,
+                                                           T *__restrict__ key_cache, T *__restrict__ value_cache,
+                                                           const Slot *__restrict__ slot_mapping, CacheGeom g) {
+  const int64_t token = blockIdx.x;
+  const int64_t pos = (int64_t)positions[token];
+  const bool rotate = pos >= 0 && pos < max_pos;
+  const int64_t slot = (int64_t)slot_mapping[token];
+  const int64_t blk = slot >= 0 ? slot / g.block_size : -1;
+  const bool cache = blk >= 0 && blk < g.num_blocks;
+  const int off = cache ? (int)(slot % g.block_size) : 0;
+  const int hd = g.head_size;
+  const int embed = rot_dim / 2;
+  const int per_head = embed / 8;
+  const T *cos_ptr = cos_sin + (rotate ? pos : 0) * rot_dim;
+  auto rotate8 = [&](T *arr, int r, uint4 &xo, uint4 &yo) {
+    const uint4 xr = *reinterpret_cast<const uint4 *>(arr + r);
+    const uint4 yr = *reinterpret_cast<const uint4 *>(arr + embed + r);
+    xo = xr;
+    yo = yr;
+    if (rotate) {
+      const uint4 cr = *reinterpret_cast<const uint4 *>(cos_ptr + r);
+      const uint4 sr = *reinterpret_cast<const uint4 *>(cos_ptr + embed + r);
+      const T *x = reinterpret_cast<const T *>(&xr), *y = reinterpret_cast<const T *>(&yr);
+      const T *c = reinterpret_cast<const T *>(&cr), *sn = reinterpret_cast<const T *>(&sr);
+      T *xe = reinterpret_cast<T *>(&xo), *ye = reinterpret_cast<T *>(&yo);
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        xe[j] = sub_t(mul_t(x[j], c[j]), mul_t(y[j], sn[j]));
+        ye[j] = add_t(mul_t(y[j], c[j]), mul_t(x[j], sn[j]));
+      }
+      *reinterpret_cast<uint4 *>(arr + r) = xo;
+      *reinterpret_cast<uint4 *>(arr + embed + r) = yo;
+    }
+  };
+  T *kc_tok = key_cache + (cache ? blk : 0) * g.k_block_stride + (int64_t)off * 8;
+  T *vc_tok = value_cache + (cache ? blk : 0) * g.v_block_stride + off;
+  const int pass_per_head = (hd - rot_dim) / 8;
+  const int n_q = num_q_heads * per_head;
+  const int n_k = g.num_heads * per_head;
+  const int n_pass = g.num_heads * pass_per_head;
+  const int n_v = g.num_heads * (hd / 8);
+  for (int i = threadIdx.x; i < n_q + n_k + n_pass + n_v; i += blockDim.x) {
+    uint4 xo, yo;
+    if (i < n_q) {
+      if (rotate) rotate8(query + token * q_stride + (int64_t)(i / per_head) * hd, (i % per_head) * 8, xo, yo);
+    } else if (i < n_q + n_k) {
+      const int j = i - n_q, h = j / per_head, r = (j % per_head) * 8;
+      rotate8(key + token * k_stride + (int64_t)h * hd, r, xo, yo);
+      if (cache) {
+        T *kc = kc_tok + h * g.k_head_stride;
+        *reinterpret_cast<uint4 *>(kc + (int64_t)(r / 8) * g.block_size * 8) = xo;
+        *reinterpret_cast<uint4 *>(kc + (int64_t)((embed + r) / 8) * g.block_size * 8) = yo;
+      }
+    } else if (i < n_q + n_k + n_pass) {
+      const int j = i - n_q - n_k, h = j / pass_per_head, ch = rot_dim / 8 + j % pass_per_head;
+      if (cache)
+        *reinterpret_cast<uint4 *>(kc_tok + h * g.k_head_stride + (int64_t)ch * g.block_size * 8) =
+            *reinterpret_cast<const uint4 *>(key + token * k_stride + (int64_t)h * hd + ch * 8);
+    } else if (cache) {
+      const int j = i - n_q - n_k - n_pass, h = j / (hd / 8), ch = j % (hd / 8);
+      const uint4 vv = *reinterpret_cast<const uint4 *>(value + token * v_tok_stride + h * v_head_stride + ch * 8);
+      const T *ve = reinterpret_cast<const T *>(&vv);
+      T *vc = vc_tok + h * g.v_head_stride + (int64_t)ch * 8 * g.block_size;
+#pragma unroll
+      for (int e = 0; e < 8; e++) vc[(int64_t)e * g.block_size] = ve[e];
+    }
+  }
+}
+
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 CacheGeom cache_geometry(const hipattn_tensor *key_cache, const hipattn_tensor *value_cache,
@@ -519,6 +599,78 @@ void cache_move(const hipattn_tensor *key, const hipattn_tensor *value,
   }
 }
 
+void take_error(char *err) {
+  if (err == nullptr) return;
+  const std::string msg(err);
+  free(err);
+  fail("%s", msg.c_str());
+}
+
+void rotary_and_cache(const hipattn_tensor *positions, hipattn_tensor *query, hipattn_tensor *key,
+                      const hipattn_tensor *value, int head_size, const hipattn_tensor *cos_sin, bool is_neox,
+                      hipattn_tensor *key_cache, hipattn_tensor *value_cache,
+                      const hipattn_tensor *slot_mapping, void *stream_arg) {
+  const char *op = "rotary_embedding_and_cache";
+  check_tensor(key, "key", 2);
+  check_tensor(query, "query", 2);
+  check_tensor(value, "value", 3);
+  check_tensor(cos_sin, "cos_sin_cache", 2);
+  check_index_tensor(positions, "positions", 1);
+  check_index_tensor(slot_mapping, "slot_mapping", 1);
+  HA_CHECK(head_size > 0 && key->sizes[1] % head_size == 0, "%s: key row width %lld is not a multiple of head_size %d", op,
+           (long long)key->sizes[1], head_size);
+  HA_CHECK(key->sizes[1] <= 1 || key->strides[1] == 1, "%s: key rows must be contiguous", op);
+  // the same key as reshape_and_cache sees it
+  hipattn_tensor key3 = *key;
+  key3.ndim = 3;
+  key3.sizes[1] = key->sizes[1] / head_size;
+  key3.sizes[2] = head_size;
+  key3.strides[1] = head_size;
+  key3.strides[2] = 1;
+  CacheGeom g = cache_geometry(key_cache, value_cache, op);
+  const int64_t T = key->sizes[0];
+  const int rot_dim = (int)cos_sin->sizes[1];
+  hipStream_t stream = resolve_stream(stream_arg);
+  const bool fused =
+      is_neox && dtype_size(key->dtype) == 2 && key->dtype == query->dtype && key->dtype == value->dtype &&
+      key->dtype == cos_sin->dtype && key->dtype == key_cache->dtype && g.head_size == head_size &&
+      key3.sizes[1] == g.num_heads && query->sizes[0] == T && value->sizes[0] == T && positions->sizes[0] == T &&
+      slot_mapping->sizes[0] == T && query->sizes[1] % head_size == 0 && (query->sizes[1] <= 1 || query->strides[1] == 1) &&
+      value->sizes[1] == g.num_heads && value->sizes[2] == head_size && (head_size <= 1 || value->strides[2] == 1) &&
+      rot_dim > 0 && rot_dim % 16 == 0 && rot_dim <= head_size && head_size % 8 == 0 && is_contiguous(cos_sin) &&
+      query->strides[0] % 8 == 0 && key->strides[0] % 8 == 0 && value->strides[0] % 8 == 0 && value->strides[1] % 8 == 0 &&
+      g.k_block_stride % 8 == 0 && g.k_head_stride % 8 == 0 && aligned16(query->data) && aligned16(key->data) &&
+      aligned16(value->data) && aligned16(cos_sin->data) && aligned16(key_cache->data) && T > 0 && T <= 0x7fffffff;
+  if (!fused) {  // every other case: the two calls, with their own checks
+    take_error(hipattn_rotary_embedding(positions, query, key, head_size, cos_sin, is_neox, stream));
+    take_error(hipattn_reshape_and_cache(&key3, value, key_cache, value_cache, slot_mapping, stream));
+    return;
+  }
+  check_data(query, "query");
+  check_data(key, "key");
+  check_data(value, "value");
+  check_data(cos_sin, "cos_sin_cache");
+  const int Hq = (int)(query->sizes[1] / head_size);
+#define HA_RC(TT, PP, SS)                                                                                            \
+  rotary_cache_kernel<TT, PP, SS><<<dim3((unsigned)T), 256, 0, stream>>>(                                             \
+      static_cast<const PP *>(positions->data), static_cast<TT *>(query->data), static_cast<TT *>(key->data),         \
+      static_cast<const TT *>(value->data), static_cast<const TT *>(cos_sin->data), rot_dim, cos_sin->sizes[0],       \
+      query->strides[0], key->strides[0], value->strides[0], value->strides[1], Hq, static_cast<TT *>(key_cache->data), \
+      static_cast<TT *>(value_cache->data), static_cast<const SS *>(slot_mapping->data), g)
+#define HA_RC_S(TT, PP)                                     \
+  if (slot_mapping->dtype == HIPATTN_I64) HA_RC(TT, PP, int64_t); \
+  else HA_RC(TT, PP, int32_t)
+#define HA_RC_P(TT)                                      \
+  if (positions->dtype == HIPATTN_I64) { HA_RC_S(TT, int64_t); } \
+  else { HA_RC_S(TT, int32_t); }
+  if (key->dtype == HIPATTN_F16) { HA_RC_P(half_t); }
+  else { HA_RC_P(bf16_t); }
+#undef HA_RC_P
+#undef HA_RC_S
+#undef HA_RC
+  check_launch(op);
+}
+
 // grid (layers, pairs): copies one block of K and of V inside every layer's
 // cache (cache_kernels.cu:55-81).
 __global__ __launch_bounds__(256) void copy_blocks_kernel(const int64_t *__restrict__ key_ptrs,
@@ -554,6 +706,15 @@ extern "C" char *hipattn_reshape_and_cache(const hipattn_tensor *key, const hipa
                                            hipattn_tensor *key_cache, hipattn_tensor *value_cache,
                                            const hipattn_tensor *slot_mapping, void *stream) {
   HA_PROTECT(cache_move<true>(key, value, key_cache, value_cache, slot_mapping, stream));
+}
+
+extern "C" char *hipattn_rotary_embedding_and_cache(const hipattn_tensor *positions, hipattn_tensor *query,
+                                                    hipattn_tensor *key, const hipattn_tensor *value, int head_size,
+                                                    const hipattn_tensor *cos_sin_cache, bool is_neox,
+                                                    hipattn_tensor *key_cache, hipattn_tensor *value_cache,
+                                                    const hipattn_tensor *slot_mapping, void *stream) {
+  HA_PROTECT(rotary_and_cache(positions, query, key, value, head_size, cos_sin_cache, is_neox, key_cache, value_cache,
+                              slot_mapping, stream));
 }
 
 extern "C" char *hipattn_gather_cached_kv(hipattn_tensor *key, hipattn_tensor *value,

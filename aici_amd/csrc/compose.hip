@@ -44,8 +44,9 @@ extern "C" char *hipattn_varlen_attn(const hipattn_tensor *q, const hipattn_tens
     HA_CHECK(q_multi >= 0 && q_multi <= T, "varlen_attn: q_multi %lld outside [0, %lld]", (long long)q_multi, (long long)T);
     const int num_kv_heads = (int)k->sizes[1];
 
-    // save_attn: every new token's K/V goes into the paged cache first (mod.rs:132-166).
-    raise(hipattn_reshape_and_cache(k, v, key_cache, value_cache, slot_mapping, stream));
+    // save_attn: every new token's K/V goes into the paged cache first (mod.rs:132-166) -- unless the
+    // caller has put it there already (hipattn_rotary_embedding_and_cache) and passes no slots.
+    if (slot_mapping) raise(hipattn_reshape_and_cache(k, v, key_cache, value_cache, slot_mapping, stream));
 
     // compute_varlen_attn (mod.rs:168-278): gather the whole context of the
     // multi-token sequences, then varlen causal attention.  The reference
@@ -88,7 +89,7 @@ extern "C" char *hipattn_varlen_attn_paged(const hipattn_tensor *q, const hipatt
     HA_CHECK(k->sizes[0] == T && v->sizes[0] == T && y->sizes[0] == T, "varlen_attn: q, k, v, y disagree on the token count");
     HA_CHECK(q_multi >= 0 && q_multi <= T, "varlen_attn: q_multi %lld outside [0, %lld]", (long long)q_multi, (long long)T);
     const int num_kv_heads = (int)k->sizes[1];
-    raise(hipattn_reshape_and_cache(k, v, key_cache, value_cache, slot_mapping, stream));
+    if (slot_mapping) raise(hipattn_reshape_and_cache(k, v, key_cache, value_cache, slot_mapping, stream));
     if (q_multi > 0) {
       HA_CHECK(multi_block_tables && multi_context_lens && seqlens_q,
                "varlen_attn: multi-token rows need their block tables, context lens and seqlens_q");

@@ -42,6 +42,24 @@ __device__ __forceinline__ T from_float(float x) {
   return (T)x;
 }
 
+// Arithmetic in T with every result rounded to T, the way the reference's per-operator half / bfloat16
+// arithmetic (and torch's CPU ops) round: no contraction into FMAs.
+template <typename T>
+__device__ __forceinline__ T mul_t(T a, T b) {
+#pragma clang fp contract(off)
+  return from_float<T>(to_float(a) * to_float(b));
+}
+template <typename T>
+__device__ __forceinline__ T add_t(T a, T b) {
+#pragma clang fp contract(off)
+  return from_float<T>(to_float(a) + to_float(b));
+}
+template <typename T>
+__device__ __forceinline__ T sub_t(T a, T b) {
+#pragma clang fp contract(off)
+  return from_float<T>(to_float(a) - to_float(b));
+}
+
 // Bit-pattern helpers for building MFMA operands out of 32-bit registers.
 template <typename V, typename U>
 __device__ __forceinline__ V bit_cast(const U &u) {

@@ -36,22 +36,6 @@ __device__ __forceinline__ float block_sum(float v, float *smem /* >= 17 floats 
 // final sum are rounded to T, which is what the reference's per-operator
 // half/bfloat16 arithmetic does and what torch's CPU ops do in the oracle.
 // ---------------------------------------------------------------------------
-template <typename T>
-__device__ __forceinline__ T mul_t(T a, T b) {
-#pragma clang fp contract(off)
-  return from_float<T>(to_float(a) * to_float(b));
-}
-template <typename T>
-__device__ __forceinline__ T add_t(T a, T b) {
-#pragma clang fp contract(off)
-  return from_float<T>(to_float(a) + to_float(b));
-}
-template <typename T>
-__device__ __forceinline__ T sub_t(T a, T b) {
-#pragma clang fp contract(off)
-  return from_float<T>(to_float(a) - to_float(b));
-}
-
 template <typename T, typename Pos, bool NEOX>
 __global__ __launch_bounds__(512) void rotary_kernel(const Pos *__restrict__ positions, T *__restrict__ query,
                                                      T *__restrict__ key, const T *__restrict__ cos_sin,

@@ -175,6 +175,17 @@ def rotary_embedding(positions: torch.Tensor, query: torch.Tensor, key: torch.Te
          int(head_size), _desc(cos_sin_cache, "cos_sin_cache"), bool(is_neox), _stream(query))
 
 
+def rotary_embedding_and_cache(positions: torch.Tensor, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                               head_size: int, cos_sin_cache: torch.Tensor, is_neox: bool, key_cache: torch.Tensor,
+                               value_cache: torch.Tensor, slot_mapping: torch.Tensor) -> None:
+    """rotary_embedding (llm/mod.rs:88-114) and reshape_and_cache (mod.rs:147-164) of a step's new tokens in
+    one launch: query/key [T, H*d] rotated in place, rotated keys and value [T, Hkv, d] written to the cache."""
+    call("hipattn_rotary_embedding_and_cache", _desc(positions, "positions"), _desc(query, "query"),
+         _desc(key, "key"), _desc(value, "value"), int(head_size), _desc(cos_sin_cache, "cos_sin_cache"),
+         bool(is_neox), _desc(key_cache, "key_cache"), _desc(value_cache, "value_cache"),
+         _desc(slot_mapping, "slot_mapping"), _stream(query))
+
+
 def rms_norm(out: torch.Tensor, input: torch.Tensor, weight: torch.Tensor, epsilon: float) -> None:
     call("hipattn_rms_norm", _desc(out, "out"), _desc(input, "input"), _desc(weight, "weight"), float(epsilon),
          _stream(input))

@@ -110,9 +110,11 @@ class Llama:
         return out
 
     def forward(self, batch_info: BatchInfo, caches: List[Tuple[torch.Tensor, torch.Tensor]],
-                paged_prefill: bool = False) -> torch.Tensor:
+                paged_prefill: bool = False, fused: bool = False) -> torch.Tensor:
         """batch_info on the device; caches[layer] = (key_cache, value_cache), updated in place.
-        paged_prefill: multi-token rows read their context through block tables (no gather copy)."""
+        paged_prefill: multi-token rows read their context through block tables (no gather copy).
+        fused: q, k, v stay views of the fused projection's output (the kernels honour the row stride) and
+        rotary + cache scatter are one launch -- four launches fewer per layer, the same bits."""
         cfg = self.cfg
         Hq, Hkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
         x = self.wte.index_select(0, batch_info.tokens.long())                   # llama.rs:203
@@ -120,9 +122,16 @@ class Llama:
         for layer, (kc, vc) in zip(self.layers, caches):
             h = self._rms(x, layer["rms_1"])                                    # :165
             qkv = h @ layer["qkv"].t()                                          # :81-83
-            q, k, v = (t.contiguous() for t in qkv.split([Hq * d, Hkv * d, Hkv * d], dim=1))
-            q, k = self.rotary.forward(batch_info.positions, q, k)              # :85 (in place on the copies)
-            y = varlen_attn(q, k, v.reshape(T, Hkv, d), batch_info, kc, vc, paged_prefill=paged_prefill)  # :93
+            if fused:
+                q, k, v = qkv.split([Hq * d, Hkv * d, Hkv * d], dim=1)
+                v = v.view(T, Hkv, d)
+                self.rotary.forward_and_cache(batch_info.positions, q, k, v, kc, vc, batch_info.slot_mapping)  # :85 + mod.rs:147-164
+                y = varlen_attn(q.view(T, Hq, d), k.view(T, Hkv, d), v, batch_info, kc, vc,
+                                paged_prefill=paged_prefill, cached=True)      # :93
+            else:
+                q, k, v = (t.contiguous() for t in qkv.split([Hq * d, Hkv * d, Hkv * d], dim=1))
+                q, k = self.rotary.forward(batch_info.positions, q, k)          # :85 (in place on the copies)
+                y = varlen_attn(q, k, v.reshape(T, Hkv, d), batch_info, kc, vc, paged_prefill=paged_prefill)  # :93
             x = y @ layer["o"].t() + x                                          # :96, :166
             h = self._rms(x, layer["rms_2"])                                    # :169
             gu = h @ layer["gate_up"].t()                                       # :135-136

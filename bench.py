@@ -249,13 +249,17 @@ def llama_step_leg(dev, stream, steps: int, layers: int, share_cache: bool) -> d
     masks = torch.from_numpy(np.packbits(np.pad(allowed, ((0, 0), (0, (-cfg.vocab_size) % 32))), axis=1,
                                          bitorder="little")).to(dev)
 
-    def step():
-        return llama.aici_greedy(model.forward(bi, caches), masks)
+    def step(fused=True):
+        return llama.aici_greedy(model.forward(bi, caches, fused=fused), masks)
 
     for _ in range(2):
         toks = step()
     torch.cuda.synchronize()
     ok = bool(torch.from_numpy(allowed)[torch.arange(S), toks.cpu().long()].all())
+    # the reference's call sequence (q, k, v copied out of the projection, rotary and cache scatter apart)
+    same = bool(torch.equal(toks, step(False)))
+    ms_ref = event_times_ms(lambda: step(False), steps, stream)
+    ms_ref = sum(ms_ref) / len(ms_ref)
     ms = event_times_ms(step, steps, stream)
     ms = sum(ms) / len(ms)
     elt = 2
@@ -268,6 +272,7 @@ def llama_step_leg(dev, stream, steps: int, layers: int, share_cache: bool) -> d
             "hbm_gbs": round((kv_bytes + weight_bytes) / (ms * 1e-3) / 1e9, 1),
             "frac_of_hbm_peak": round((kv_bytes + weight_bytes) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "constrained_tokens_all_allowed": ok,
+            "ms_per_step_reference_call_sequence": round(ms_ref, 3), "same_tokens_either_way": same,
             "config": {"workload": f"Llama-3-8B-shaped decode step, {layers} layers, 128 seqs, ctx U[1024,16384] "
                                    "(seed 5), bf16, per-layer paged KV"
                                    + (" (one cache shared by all layers)" if share_cache else "")

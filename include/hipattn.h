@@ -197,6 +197,21 @@ char *hipattn_rotary_embedding(const hipattn_tensor *positions,
                                const hipattn_tensor *cos_sin_cache,
                                bool is_neox, void *stream);
 
+/* hipattn_rotary_embedding followed by hipattn_reshape_and_cache of the same
+ * keys, in one launch: what a layer does with a step's new tokens
+ * (llm/mod.rs:88-114 then 147-164).  No counterpart in the reference's FFI;
+ * same results as the two calls, bit for bit.  query [T, Hq*d] and key
+ * [T, Hkv*d] are rotated in place, the rotated keys and value [T, Hkv, d] go to
+ * the slots of slot_mapping (int64 or int32; negative = not cached).  NeoX
+ * layout on a 2-byte type takes the fused kernel; anything else runs the two
+ * calls one after the other. */
+char *hipattn_rotary_embedding_and_cache(
+    const hipattn_tensor *positions, hipattn_tensor *query, hipattn_tensor *key,
+    const hipattn_tensor *value, int head_size,
+    const hipattn_tensor *cos_sin_cache, bool is_neox,
+    hipattn_tensor *key_cache, hipattn_tensor *value_cache,
+    const hipattn_tensor *slot_mapping, void *stream);
+
 /* Replaces rms_norm_C (lib.rs:139-144; layernorm_kernels.cu:10-35,69-92). */
 char *hipattn_rms_norm(hipattn_tensor *out, const hipattn_tensor *input,
                        const hipattn_tensor *weight, float epsilon,
@@ -463,7 +478,9 @@ int64_t hipattn_cache_block_bytes(int64_t block_size, int64_t num_kv_heads,
  * int32 [G], seqlens_q/k int32 [num_multi+1], paged_block_tables,
  * paged_context_lens.  gather_k/gather_v [G, Hkv, d] are scratch for the
  * gathered context.  The GQA head mapping is done inside the kernels; no
- * repeat_kv copy (mod.rs:357-365) is made. */
+ * repeat_kv copy (mod.rs:357-365) is made.  slot_mapping NULL = the new K/V are
+ * in the cache already (hipattn_rotary_embedding_and_cache put them there) and
+ * the scatter is skipped; the same holds for hipattn_varlen_attn_paged. */
 char *hipattn_varlen_attn(
     const hipattn_tensor *q, const hipattn_tensor *k, const hipattn_tensor *v,
     hipattn_tensor *key_cache, hipattn_tensor *value_cache,

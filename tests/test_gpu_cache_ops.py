@@ -273,3 +273,45 @@ def test_swapped_out_sequence_decodes_the_same_after_swap_in(device):
     after, blocks_after = decode()
     assert blocks_after != blocks_before
     assert torch.equal(bits(after), bits(before))
+
+
+@pytest.mark.parametrize("case", [
+    (torch.bfloat16, 32, 8, 128, 128, True, torch.int64),    # Llama: the fused kernel
+    (torch.float16, 32, 32, 80, 32, True, torch.int32),      # Phi-2: rot_dim < d, pass-through chunks
+    (torch.float16, 8, 2, 64, 64, False, torch.int64),       # GPT-J pairing: the two calls behind the entry point
+    (torch.float32, 4, 4, 64, 64, True, torch.int64),        # fp32: likewise
+    (torch.bfloat16, 4, 1, 96, 48, True, torch.int64),       # rot_dim not a multiple of 16: likewise
+])
+def test_rotary_and_cache_equals_the_two_calls(device, case):
+    """hipattn_rotary_embedding_and_cache against the oracle's rotary_embedding + reshape_and_cache, bit for
+    bit, on strided q/k/v (chunks of one fused QKV row), with padding slots, a slot past the cache and
+    positions outside the table."""
+    dtype, Hq, Hkv, d, rot, neox, slot_dtype = case
+    g = torch.Generator().manual_seed(41)
+    T, bs, nb, max_pos = 150, 16, 24, 500
+    qkv = torch.randn((T, (Hq + 2 * Hkv) * d), generator=g).to(dtype)
+    q, k, v = qkv[:, :Hq * d], qkv[:, Hq * d:(Hq + Hkv) * d], qkv[:, (Hq + Hkv) * d:].view(T, Hkv, d)
+    pos = torch.randint(0, max_pos, (T,), generator=g)
+    pos[7], pos[8] = max_pos + 3, -1                       # outside the table: rows left as they are
+    slots = torch.randperm(nb * bs, generator=g)[:T].to(torch.int64)
+    slots[11], slots[12] = -1, nb * bs + 5                 # not cached
+    table = ref.rotary_table(rot, 10000.0, max_pos, dtype)
+    kc, vc = make_cache(nb, Hkv, d, bs, dtype, fill=-2.0)
+    # oracle: rotate (valid positions only), then scatter (valid slots only)
+    q_ref, k_ref = q.clone(), k.clone()
+    okp = (pos >= 0) & (pos < max_pos)
+    qr, kr = q_ref[okp].clone(), k_ref[okp].clone()
+    ref.rotary_embedding(pos[okp], qr, kr, d, table, neox)
+    q_ref[okp], k_ref[okp] = qr, kr
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    oks = (slots >= 0) & (slots < nb * bs)
+    ref.reshape_and_cache(k_ref.view(T, Hkv, d)[oks], v[oks], kc_ref, vc_ref, slots[oks])
+    qkv_d = qkv.to(device)
+    qd, kd = qkv_d[:, :Hq * d], qkv_d[:, Hq * d:(Hq + Hkv) * d]
+    vd = qkv_d[:, (Hq + Hkv) * d:].view(T, Hkv, d)
+    kcd, vcd = kc.to(device), vc.to(device)
+    K.rotary_embedding_and_cache(pos.to(device), qd, kd, vd, d, table.to(device), neox, kcd, vcd,
+                                 slots.to(slot_dtype).to(device))
+    assert torch.equal(bits(qd), bits(q_ref)) and torch.equal(bits(kd), bits(k_ref))
+    assert torch.equal(bits(kcd), bits(kc_ref)) and torch.equal(bits(vcd), bits(vc_ref))
+    assert torch.equal(bits(vd), bits(v))

@@ -71,9 +71,9 @@ class TwoSides:
         return b.finish(), hostkv.build_batch(entries, 16, self.cfg.max_position_embeddings, 0)
 
 
-@pytest.mark.parametrize("paged_prefill", [False, True])
+@pytest.mark.parametrize("paged_prefill,fused", [(False, False), (True, False), (False, True), (True, True)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_three_steps_match_the_cpu_build(device, dtype, paged_prefill):
+def test_three_steps_match_the_cpu_build(device, dtype, paged_prefill, fused):
     cfg = make_cfg(dtype)
     ws = llama.random_weights(cfg, seed=5, std=0.04)
     model = llama.Llama(cfg, ws, device)
@@ -85,7 +85,7 @@ def test_three_steps_match_the_cpu_build(device, dtype, paged_prefill):
 
     def run(order):
         bi_g, bi_c = sides.step(order)
-        got = model.forward(bi_g.to(device), sides.caches_g, paged_prefill=paged_prefill).float().cpu()
+        got = model.forward(bi_g.to(device), sides.caches_g, paged_prefill=paged_prefill, fused=fused).float().cpu()
         want = ollama.forward(cfg, ws, bi_c, sides.caches_c, cos_sin)
         # the GPU batch puts multi-token entries first; line rows up by sequence id
         row = {sid: i for i, sid in enumerate(bi_g.seq_ids)}
