@@ -131,3 +131,46 @@ def test_argument_errors(device):
     big = paged_case(35, [(0, 4)], 2, 2, 256, torch.float16, 4)
     with pytest.raises(HipAttnError, match="head size"):
         run_paged(big, device)
+
+
+def test_blocks_beyond_4_gib_of_cache(device):
+    """A cache of 4.6 GB per tensor whose used blocks lie past the 4 GiB mark: block offsets need 64 bits in
+    the scatter, in both paged prefill forms and in the decode kernel.  Checked against the library's own
+    gather + contiguous prefill on the same cache (itself checked against the oracle above)."""
+    dtype, Hq, Hkv, d, bs = torch.bfloat16, 16, 8, 128, 16
+    nb = 140000                                           # x 32 KiB per block = 4.59 GB each for K and V
+    kc = torch.zeros((nb, Hkv, d // 8, bs, 8), dtype=dtype, device=device)
+    vc = torch.zeros((nb, Hkv, d, bs), dtype=dtype, device=device)
+    g = torch.Generator().manual_seed(35)
+    seqs = [(1500, 300), (0, 700), (40, 1)]
+    lens_k, lens_q = [a + b for a, b in seqs], [b for _, b in seqs]
+    high = (136000 + torch.randperm(4000, generator=g)).tolist()      # byte offsets from 4.45 GB up
+    width = max((l + 15) // 16 for l in lens_k)
+    tables = torch.zeros((len(seqs), width), dtype=torch.int32)
+    slots = []
+    for i, lk in enumerate(lens_k):
+        n = (lk + 15) // 16
+        blocks = [high.pop() for _ in range(n)]
+        tables[i, :n] = torch.tensor(blocks, dtype=torch.int32)
+        slots += W.slots_for(blocks, lk)
+    k = torch.randn((sum(lens_k), Hkv, d), generator=g).to(dtype).to(device)
+    v = torch.randn((sum(lens_k), Hkv, d), generator=g).to(dtype).to(device)
+    q = torch.randn((sum(lens_q), Hq, d), generator=g).to(dtype).to(device)
+    slots_d = torch.tensor(slots, dtype=torch.int64, device=device)
+    K.reshape_and_cache(k, v, kc, vc, slots_d)
+    gk, gv = torch.empty_like(k), torch.empty_like(v)
+    K.gather_cached_kv(gk, gv, kc, vc, slots_d.to(torch.int32))
+    assert torch.equal(gk, k) and torch.equal(gv, v)
+    cu_q, cu_k = W.offsets(lens_q).to(device), W.offsets(lens_k).to(device)
+    ctx = torch.tensor(lens_k, dtype=torch.int32, device=device)
+    scale = 1.0 / math.sqrt(d)
+    want = K.flash_attn_varlen(q, k, v, cu_q, cu_k, max(lens_q), max(lens_k), scale, True)
+    got = K.flash_attn_varlen_paged(q, kc, vc, tables.to(device), cu_q, ctx, max(lens_q), max(lens_k), scale, True)
+    assert (got.float() - want.float()).abs().max().item() <= TOL[dtype]
+    # decode rows over the same contexts: equal to the last row of a prefill over the whole context
+    qd = torch.randn((len(seqs), Hq, d), generator=g).to(dtype).to(device)
+    out = torch.empty_like(qd)
+    K.paged_attention_v1(out, qd, kc, vc, Hkv, scale, tables.to(device), ctx, 16, max(lens_k))
+    one = W.offsets([1] * len(seqs)).to(device)
+    want_d = K.flash_attn_varlen(qd, k, v, one, cu_k, 1, max(lens_k), scale, True)
+    assert (out.float() - want_d.float()).abs().max().item() <= TOL[dtype]
