@@ -836,6 +836,7 @@ GenericDecodeParams generic_params(const DecodeParams &p, int head_size, int blo
   g.num_blocks = p.num_blocks;
   g.block_tables = p.block_tables;
   g.table_stride = p.max_blocks;
+  g.table_cols = p.table_cols;
   g.context_lens = p.context_lens;
   g.alibi = p.alibi;
   g.scale = scale;

@@ -17,6 +17,7 @@ struct GenericDecodeParams {
   int64_t num_blocks;
   const int32_t *block_tables;
   int64_t table_stride;
+  int table_cols;  // columns of block_tables: lookups are clamped to them
   const int32_t *context_lens;
   const float *alibi;  // [Hq] or null
   float scale;

@@ -65,7 +65,8 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(GenericDecode
   const int qh = blockIdx.x, seq = blockIdx.y, part = blockIdx.z;
   const int tid = threadIdx.x;
   const int hd = p.head_size;
-  const int ctx = p.context_lens[seq];
+  // a context cannot be longer than its table row can describe
+  const int ctx = min(p.context_lens[seq], p.table_cols * BS);
   const int t0 = part * p.part_tokens;
   T *op = static_cast<T *>(p.out) + seq * p.out_stride + (int64_t)qh * hd;
   if (t0 >= ctx) {
@@ -172,7 +173,7 @@ __global__ __launch_bounds__(64) void paged_decode_generic_reduce_kernel(Generic
   const int qh = blockIdx.x, seq = blockIdx.y;
   const int lane = threadIdx.x;
   const int hd = p.head_size;
-  const int ctx = p.context_lens[seq];
+  const int ctx = min(p.context_lens[seq], p.table_cols * p.block_size);
   if (ctx <= 0) return;  // the main kernel wrote the zero row
   const int np = (ctx + p.part_tokens - 1) / p.part_tokens;
   const int64_t base = ((int64_t)seq * p.Hq + qh) * p.num_parts;
