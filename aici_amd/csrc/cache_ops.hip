@@ -191,7 +191,7 @@ __global__ __launch_bounds__(256) void cache_move_run8_kernel(
 // above; groups that are not a run of 8 slots take its per-token path, and a workgroup whose 16 tokens
 // fill one whole block moves 16-token tiles, whose cache side is whole rows ([chunk][16 tokens] = 256
 // bytes of K, [16 tokens] = 32 bytes of each V element, 1 KiB contiguous per instruction).
-template <typename Slot, bool SCATTER>
+template <typename Slot, bool SCATTER, bool FULL_GROUPS>
 __global__ __launch_bounds__(256) void cache_move_tile_kernel(
     uint16_t *__restrict__ key, uint16_t *__restrict__ value, uint16_t *__restrict__ key_cache,
     uint16_t *__restrict__ value_cache, const Slot *__restrict__ slot_mapping, int64_t num_tokens,
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
     const int64_t blk = run_slot[0] / 16;
     for (int item = wave; item < items_per_half; item += 4) {
       const int h = item / groups_per_head, cg = item % groups_per_head;
-      const int nc = min(8, chunks_per_head - 8 * cg);  // chunks in this group
+      const int nc = FULL_GROUPS ? 8 : min(8, chunks_per_head - 8 * cg);  // chunks in this group
       E *kc_base = key_cache + blk * g.k_block_stride + h * g.k_head_stride;
       E *vc_base = value_cache + blk * g.v_block_stride + h * g.v_head_stride;
       const int tok = lane & 15, c4 = lane >> 4;
@@ -310,7 +310,7 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
       E *v_tok = value + (t0 + hi) * val_tok_stride + h * val_head_stride + (cg * 8 + lo) * X;
       E *k_cache = kc_base + ((int64_t)(cg * 8 + hi) * g.block_size + off0 + lo) * X;
       E *v_cache = vc_base + (int64_t)((cg * 8 + hi) * X + lo) * g.block_size + off0;
-      const int nc = min(8, chunks_per_head - 8 * cg);  // chunks in this group
+      const int nc = FULL_GROUPS ? 8 : min(8, chunks_per_head - 8 * cg);  // chunks in this group
       if (SCATTER) {
         if (lo < nc) {
           *reinterpret_cast<uint4 *>(ks + hi * KP + lo * X) = *reinterpret_cast<const uint4 *>(k_tok);
@@ -351,7 +351,7 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
       const int64_t blk = slot / g.block_size;
       if (blk >= g.num_blocks) continue;
       const int off = (int)(slot % g.block_size);
-      if (lane < min(8, chunks_per_head - 8 * cg)) {
+      if (lane < (FULL_GROUPS ? 8 : min(8, chunks_per_head - 8 * cg))) {
         const int c = cg * 8 + lane;
         E *kp = key + token * key_tok_stride + h * key_head_stride + c * X;
         E *vp = value + token * val_tok_stride + h * val_head_stride + c * X;
@@ -532,8 +532,13 @@ void launch_move(const hipattn_tensor *key, const hipattn_tensor *value,
       // The LDS-transposing kernel pays off (whole rows on both sides) once there are enough 16-token
       // workgroups to hide its load -> LDS -> store chains.
       if (T >= 16384 && getenv("HIPATTN_CACHE_MOVE_NO_LDS") == nullptr) {
-        cache_move_tile_kernel<Slot, SCATTER><<<dim3((unsigned)((T + 15) / 16)), 256, 0, stream>>>(
-            kp, vp, kc, vc, sp, T, key->strides[0], key->strides[1], value->strides[0], value->strides[1], g);
+        // head sizes that are multiples of 64 have no partial chunk group: their instance carries no guards
+        if (g.head_size % 64 == 0)
+          cache_move_tile_kernel<Slot, SCATTER, true><<<dim3((unsigned)((T + 15) / 16)), 256, 0, stream>>>(
+              kp, vp, kc, vc, sp, T, key->strides[0], key->strides[1], value->strides[0], value->strides[1], g);
+        else
+          cache_move_tile_kernel<Slot, SCATTER, false><<<dim3((unsigned)((T + 15) / 16)), 256, 0, stream>>>(
+              kp, vp, kc, vc, sp, T, key->strides[0], key->strides[1], value->strides[0], value->strides[1], g);
         check_launch(SCATTER ? "reshape_and_cache" : "gather_cached_kv");
         return;
       }
