@@ -1278,10 +1278,10 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
 template <typename T>
 void dispatch_paged(const PrefillParams &p, hipStream_t stream) {
   const int hdp = ((p.d + 31) / 32) * 32;
-  // Head sizes that fill their MFMA tiles take the block images as they are; the others are staged
-  // through registers, which pads them.  HIPATTN_PAGED_PREFILL_DMA=0 forces the staged form (tuning aid).
+  // Head sizes that fill their MFMA tiles take the block images as they are (16-byte aligned images); the
+  // others are staged through registers, which pads them.  HIPATTN_PAGED_PREFILL_DMA=0 forces the staged form (tuning aid).
   const char *force = getenv("HIPATTN_PAGED_PREFILL_DMA");
-  const bool dma = p.d == hdp && !(force && force[0] == '0');
+  const bool dma = p.d == hdp && p.vc_block % 8 == 0 && p.vc_head % 8 == 0 && !(force && force[0] == '0');
 #define HA_W8P(H)                                              \
   if (dma) launch_prefill_w8<T, H, W8_PAGED_DMA>(p, stream);   \
   else launch_prefill_w8<T, H, W8_PAGED>(p, stream)
