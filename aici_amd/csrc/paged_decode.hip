@@ -363,38 +363,64 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(DecodeParams p) {
   }
 }
 
-// Merge of the partitions of one (sequence, query head): grid (Hq, S), one
-// wavefront per 64 head elements.  Lane i first owns partition i's (max, sum)
-// to form the weights, then every lane owns one head element.
-template <typename T, int HD, bool V2FMT>
-__global__ __launch_bounds__(256) void paged_decode_reduce_kernel(DecodeParams p) {
+// Merge of the partitions of one (sequence, query head): grid (Hq, S).  A long context of a small batch
+// is cut into hundreds of partitions (the main launch wants a few thousand workgroups), so the merge is
+// spread over the workgroup: thread (slice, d) sums the partitions slice, slice + SLICES, ... of head element
+// d, four loads in flight, and the slices meet in LDS (one slice when there are few partitions).
+template <typename T, int HD, bool V2FMT, int THREADS>
+__global__ __launch_bounds__(THREADS) void paged_decode_reduce_kernel(DecodeParams p) {
+  constexpr int HDT = HD <= 64 ? 64 : (HD <= 128 ? 128 : 256);  // threads per slice
+  static_assert(THREADS % HDT == 0 && THREADS % 64 == 0, "whole slices, whole wavefronts");
+  constexpr int SLICES = THREADS / HDT;
+  constexpr int WAVES = THREADS / 64;
+  __shared__ float s_red[WAVES];
+  __shared__ float s_o[SLICES][HDT];
   const int qh = blockIdx.x, seq = blockIdx.y;
-  const int lane = threadIdx.x & 63;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ctx = p.context_lens[seq];
   const int nblk = (ctx + kBlockSize - 1) / kBlockSize;
   const int np = (nblk + p.part_blocks - 1) / p.part_blocks;  // partitions that ran
   const int64_t base = ((int64_t)seq * p.Hq + qh) * p.num_parts;
   T *op = static_cast<T *>(p.out) + seq * p.out_stride + (int64_t)qh * HD;
   const float mscale = V2FMT ? kLog2e : 1.0f;  // v2 maxima are natural-log
+  auto block_reduce = [&](float v, bool is_max) -> float {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float t = __shfl_xor(v, o, 64);
+      v = is_max ? fmaxf(v, t) : v + t;
+    }
+    __syncthreads();  // s_red may still be read from the previous reduction
+    if (lane == 0) s_red[wave] = v;
+    __syncthreads();
+    v = s_red[0];
+#pragma unroll
+    for (int i = 1; i < WAVES; i++) v = is_max ? fmaxf(v, s_red[i]) : v + s_red[i];
+    return v;
+  };
   float mmax = -INFINITY;
-  for (int i = lane; i < np; i += 64) mmax = fmaxf(mmax, p.ws_m[base + i] * mscale);
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) mmax = fmaxf(mmax, __shfl_xor(mmax, o, 64));
+  for (int i = tid; i < np; i += THREADS) mmax = fmaxf(mmax, p.ws_m[base + i] * mscale);
+  mmax = block_reduce(mmax, true);
   float denom = 0.f;
-  for (int i = lane; i < np; i += 64) denom += p.ws_l[base + i] * fast_exp2(p.ws_m[base + i] * mscale - mmax);
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) denom += __shfl_xor(denom, o, 64);
+  for (int i = tid; i < np; i += THREADS) denom += p.ws_l[base + i] * fast_exp2(p.ws_m[base + i] * mscale - mmax);
+  denom = block_reduce(denom, false);
   const float inv = denom > 0.f ? 1.0f / denom : 0.f;
-  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
-    float o = 0.f;
+  const int slice = tid / HDT, d = tid % HDT;
+  float o = 0.f;
+  if (d < HD) {
 #pragma unroll 4
-    for (int i = 0; i < np; i++) {
+    for (int i = slice; i < np; i += SLICES) {
       const float w = fast_exp2(p.ws_m[base + i] * mscale - mmax);
       if (V2FMT)
         o += to_float(static_cast<const T *>(p.tmp_out)[(base + i) * HD + d]) * (w * p.ws_l[base + i]);
       else
         o += p.ws_acc[(base + i) * HD + d] * w;
     }
+  }
+  s_o[slice][d] = o;
+  __syncthreads();
+  if (slice == 0 && d < HD) {
+#pragma unroll
+    for (int k = 1; k < SLICES; k++) o += s_o[k][d];
     op[d] = from_float<T>(o * inv);
   }
 }
@@ -407,7 +433,12 @@ void launch_decode(const DecodeParams &p, int64_t S, hipStream_t stream) {
   paged_decode_kernel<T, HD, V2FMT><<<grid, 256, 0, stream>>>(p);
   check_launch("paged_attention");
   if (p.num_parts > 1) {
-    paged_decode_reduce_kernel<T, HD, V2FMT><<<dim3((unsigned)p.Hq, (unsigned)S), HD <= 64 ? 64 : 128, 0, stream>>>(p);
+    // few partitions: one slice of threads is enough and cheaper to start
+    if (p.num_parts <= 8)
+      paged_decode_reduce_kernel<T, HD, V2FMT, (HD <= 64 ? 64 : (HD <= 128 ? 128 : 256))>
+          <<<dim3((unsigned)p.Hq, (unsigned)S), HD <= 64 ? 64 : (HD <= 128 ? 128 : 256), 0, stream>>>(p);
+    else
+      paged_decode_reduce_kernel<T, HD, V2FMT, 512><<<dim3((unsigned)p.Hq, (unsigned)S), 512, 0, stream>>>(p);
     check_launch("paged_attention reduce");
   }
 }
