@@ -3,14 +3,14 @@
 // 447-655 and flash_fwd_kernel.h:590-1136) with a design laid out for CDNA4.
 // Two kernels share the mathematics:
 //
-//  * prefill_varlen_w8_kernel (head sizes up to 128, launches of a few hundred
-//    workgroups or more): 8 wavefronts own 256 query rows, two per SIMD, each
+//  * prefill_varlen_w8_kernel (head sizes up to 128, causal or unmasked): 8
+//    wavefronts own 256 query rows, two per SIMD, each
 //    running one software-pipelined loop over 64-key tiles held in three LDS
 //    buffers, V stored transposed in LDS; two more instances read K/V from the
 //    paged cache through block tables -- staged through registers like the
 //    rows, or, for head sizes that fill their MFMA tiles, copied into LDS block
 //    by block with global -> LDS loads.  Described at its definition.
-//  * prefill_varlen_kernel (small launches, head sizes up to 256): a workgroup
+//  * prefill_varlen_kernel (head sizes up to 256, sliding windows): a workgroup
 //    of 4 wavefronts owns 128 or 256 query rows of one (sequence, query head);
 //    each wavefront keeps QT tiles of 32 query rows, their Q operands and their
 //    fp32 output accumulators in registers; K and V tiles of 64 keys are staged
@@ -1117,17 +1117,17 @@ void launch_prefill(PrefillParams p, hipStream_t stream) {
 
 template <typename T, int HDP>
 void pick_qt(const PrefillParams &p, int64_t total_q, hipStream_t stream) {
-  // The eight-wavefront kernel (256-row workgroups) wins from a few hundred workgroups up -- measured
-  // 4 x 512 tokens x 32 heads: 28 vs 33 us, 2 x 2048: 90 vs 144 us; only the smallest launches (4 sequences
-  // of 128..512 tokens: 24.6 vs 22.7 us) prefer 128-row workgroups.
+  // The eight-wavefront kernel (256-row workgroups) is at least as fast at every launch size measured -- 4
+  // sequences of 128..512 tokens x 32 heads: 21.6 vs 23.3 us, 4 x 512: 25 vs 36 us, 2 x 2048: 85 vs 152 us; one
+  // 128-token sequence: 17 us either way -- so the four-wavefront kernel is left with what the other does not
+  // do: head sizes above 128, sliding windows, rows too far apart for 32-bit offsets.
   if constexpr (HDP <= 128) {
-    const int64_t wg256 = (total_q / 256 + p.batch) * p.Hq;
     const char *force = getenv("HIPATTN_PREFILL_KERNEL");  // tuning aid: "w8", "qt2" or "qt1"
     // the eight-wavefront kernel addresses a tile's 64 rows with 32-bit byte offsets
-    const bool big = wg256 >= 320 && p.k_row < (1 << 23) && p.v_row < (1 << 23);
+    const bool fits = p.k_row < (1 << 23) && p.v_row < (1 << 23);
     // it knows the causal mask and no mask; other windows go to the four-wavefront kernel
     const bool plain = p.win_left < 0 && p.win_right <= 0;
-    if (plain && (force ? !strcmp(force, "w8") : big) && p.k_row < (1 << 23) && p.v_row < (1 << 23)) {
+    if (plain && fits && (force ? !strcmp(force, "w8") : true)) {
       launch_prefill_w8<T, HDP>(p, stream);
       return;
     }
