@@ -262,6 +262,25 @@ def llama_step_leg(dev, stream, steps: int, layers: int, share_cache: bool) -> d
     ms_ref = sum(ms_ref) / len(ms_ref)
     ms = event_times_ms(step, steps, stream)
     ms = sum(ms) / len(ms)
+    # the same step captured once in a HIP graph and replayed: no launch gaps between its ~400 kernels
+    ms_graph, same_graph = None, None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            toks_graph = step()
+        graph.replay()
+        torch.cuda.synchronize()
+        same_graph = bool(torch.equal(toks_graph, toks))
+        ms_graph = event_times_ms(graph.replay, steps, stream)
+        ms_graph = round(sum(ms_graph) / len(ms_graph), 3)
+    except Exception as e:  # reported, not fatal: the eager figures above stand on their own
+        ms_graph = f"capture failed: {type(e).__name__}: {e}"[:200]
     elt = 2
     kv_bytes = int(ctx.sum()) * 2 * cfg.num_key_value_heads * cfg.head_dim * elt * layers
     H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
@@ -273,6 +292,7 @@ def llama_step_leg(dev, stream, steps: int, layers: int, share_cache: bool) -> d
             "frac_of_hbm_peak": round((kv_bytes + weight_bytes) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "constrained_tokens_all_allowed": ok,
             "ms_per_step_reference_call_sequence": round(ms_ref, 3), "same_tokens_either_way": same,
+            "ms_per_step_hip_graph_replay": ms_graph, "same_tokens_from_graph": same_graph,
             "config": {"workload": f"Llama-3-8B-shaped decode step, {layers} layers, 128 seqs, ctx U[1024,16384] "
                                    "(seed 5), bf16, per-layer paged KV"
                                    + (" (one cache shared by all layers)" if share_cache else "")
