@@ -78,6 +78,9 @@ _ERR_FUNCS = {
                                TP, TP, c_void_p],
     "hipattn_mha_varlen_fwd_paged": [TP, TP, TP, TP, TP, TP, c_int, c_int, c_float, c_bool, TP, TP, c_void_p],
     "hipattn_paged_attention_v1": [TP, TP, TP, TP, c_int, c_float, TP, TP, c_int, c_int, TP, c_void_p],
+    "hipattn_paged_attention_v1_ws": [TP, TP, TP, TP, c_int, c_float, TP, TP, c_int, c_int, TP, c_void_p, c_int64,
+                                      c_void_p],
+    "hipattn_paged_attention_workspace_size": [c_int64, c_int, c_int, c_int, c_int, c_int, c_int32, POINTER(c_int64)],
     "hipattn_paged_attention_v2": [TP, TP, TP, TP, TP, TP, TP, c_int, c_float, TP, TP, c_int, c_int, TP, c_void_p],
     "hipattn_reshape_and_cache": [TP, TP, TP, TP, TP, c_void_p],
     "hipattn_gather_cached_kv": [TP, TP, TP, TP, TP, c_void_p],
@@ -113,6 +116,8 @@ _ERR_FUNCS = {
     "hipattn_event_synchronize": [c_void_p],
     "hipattn_event_free": [c_void_p],
     "hipattn_shutdown": [],
+    "hipattn_tuning_set": [c_char_p, c_int],
+    "hipattn_tuning_get": [c_char_p, POINTER(c_int)],
     "hipattn_block_allocator_new": [c_int64, c_int64, POINTER(c_void_p)],
     "hipattn_block_allocator_alloc_seq": [c_void_p, c_int64, c_int64],
     "hipattn_block_allocator_set_watermark": [c_void_p, ctypes.c_float],

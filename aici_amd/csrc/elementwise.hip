@@ -683,7 +683,7 @@ void bias_argmax_impl(const hipattn_tensor *logits, const hipattn_tensor *bias, 
     if (chunks < 1) chunks = 1;
     const int per_slice = (int)((((V + chunks - 1) / chunks) + 7) / 8 * 8);
     chunks = (V + per_slice - 1) / per_slice;
-    char *ws = static_cast<char *>(library_workspace((size_t)S * chunks * 8, stream));
+    char *ws = static_cast<char *>(library_workspace(WS_BIAS_ARGMAX, (size_t)S * chunks * 8, stream));
     float *pv = reinterpret_cast<float *>(ws);
     int32_t *pi = reinterpret_cast<int32_t *>(ws + (size_t)S * chunks * 4);
     const dim3 grid((unsigned)chunks, (unsigned)S);

@@ -25,6 +25,9 @@
 // exp2((s - max) * log2e-folded scale), rounded to the cache dtype only as the
 // MFMA operand of P.V; the normaliser is the fp32 sum of the unrounded
 // probabilities.
+#include <algorithm>
+#include <atomic>
+
 #include "common.h"
 #include "device_types.h"
 #include "paged_decode_generic.h"
@@ -63,10 +66,11 @@ struct DecodeParams {
   void *tmp_out;  // [S, Hq, P, HD] in T (reference v2 format)
   void *out;      // [S, Hq, HD]
   int64_t out_stride;
+  int max_ctx;  // context lengths are clamped to this (the caller's max_context_len, at most what a table row holds)
   // flat split (paged_decode_flat_kernel)
   int *flat_prefix;  // [S + 1] block pairs before each sequence, written by workgroup 0
   int flat_waves;    // wavefronts of the main launch
-  int flat_cols;     // query-head columns kept per partial slot: min(G, 16)
+  int flat_cols;   // query-head columns kept per partial slot: min(G, 16)
 };
 
 template <typename T>
@@ -248,7 +252,7 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(DecodeParams p) {
   const int b0 = part * p.part_blocks;
   int tbl = 0;
   if (lane < p.part_blocks && b0 + lane < p.table_cols) tbl = p.block_tables[seq * p.max_blocks + b0 + lane];
-  const int ctx = p.context_lens[seq];
+  const int ctx = min(p.context_lens[seq], p.max_ctx);
   const int nblk = (ctx + kBlockSize - 1) / kBlockSize;
   const int g_idx = cg * 16 + col;  // query head within the GQA group
   const bool col_ok = g_idx < p.G;
@@ -377,7 +381,7 @@ __global__ __launch_bounds__(THREADS) void paged_decode_reduce_kernel(DecodePara
   __shared__ float s_o[SLICES][HDT];
   const int qh = blockIdx.x, seq = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int ctx = p.context_lens[seq];
+  const int ctx = min(p.context_lens[seq], p.max_ctx);
   const int nblk = (ctx + kBlockSize - 1) / kBlockSize;
   const int np = (nblk + p.part_blocks - 1) / p.part_blocks;  // partitions that ran
   const int64_t base = ((int64_t)seq * p.Hq + qh) * p.num_parts;
@@ -514,7 +518,7 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void paged_decode_flat_kern
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const int s = 4 * tid + j;
-      c[j] = s < S ? p.context_lens[s] : 0;
+      c[j] = s < S ? min(p.context_lens[s], p.max_ctx) : 0;
       n[j] = ctx_pairs(c[j]);
       tsum += n[j];
     }
@@ -753,80 +757,65 @@ __global__ __launch_bounds__(128) void paged_decode_flat_reduce_kernel(DecodePar
   }
 }
 
-// Workgroups of the flat launch: what the device holds at once (times a small
-// oversubscription factor), but no more than gives every wavefront
-// `min_chunk` units of the largest possible step.
+// Workgroups of the flat kernel that the device holds at once, per device (asked of the runtime once).
 template <typename T, int HD>
-int flat_workgroups(int64_t max_units) {
-  static int resident = 0;  // workgroups of this kernel the current device holds
-  if (resident == 0) {
-    int dev = 0, per_cu = 0;
-    hipDeviceProp_t prop;
-    HA_HIP(hipGetDevice(&dev));
-    HA_HIP(hipGetDeviceProperties(&prop, dev));
+int flat_resident_workgroups() {
+  constexpr int kDevices = 64;
+  static std::atomic<int> resident[kDevices];
+  int dev = 0;
+  HA_HIP(hipGetDevice(&dev));
+  HA_CHECK(dev >= 0 && dev < kDevices, "device index %d out of range", dev);
+  int r = resident[dev].load(std::memory_order_relaxed);
+  if (r == 0) {
+    int per_cu = 0, cus = 0;
+    HA_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     HA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, paged_decode_flat_kernel<T, HD>, 256, 0));
-    resident = (per_cu > 0 ? per_cu : 1) * prop.multiProcessorCount;
+    r = (per_cu > 0 ? per_cu : 1) * (cus > 0 ? cus : 1);
+    resident[dev].store(r, std::memory_order_relaxed);
   }
-  int64_t wgs = resident;
-  if (const char *e = getenv("HIPATTN_DECODE_FLAT_WGS")) {
-    const int v = atoi(e);
-    if (v > 0) wgs = v;
-  }
-  const int64_t min_chunk = 2;
-  const int64_t cap = (max_units + 4 * min_chunk - 1) / (4 * min_chunk);
-  if (wgs > cap) wgs = cap;
-  return (int)(wgs < 1 ? 1 : wgs);
+  return r;
 }
 
-template <typename T, int HD>
-void launch_decode_flat(DecodeParams p, int64_t S, int max_context_len, hipStream_t stream) {
-  const int64_t max_units = S * p.Hkv * p.col_groups * ((max_context_len + 2 * kBlockSize - 1) / (2 * kBlockSize));
-  const int wgs = flat_workgroups<T, HD>(max_units);
-  p.flat_waves = wgs * 4;
-  p.flat_cols = p.G < 16 ? p.G : 16;
-  const size_t slots = (size_t)2 * p.flat_waves * p.flat_cols;
-  const size_t prefix_bytes = (((size_t)S + 1) * sizeof(int) + 255) & ~(size_t)255;
-  char *ws = static_cast<char *>(library_workspace(prefix_bytes + slots * (HD + 2) * sizeof(float), stream));
-  p.flat_prefix = reinterpret_cast<int *>(ws);
-  p.ws_acc = reinterpret_cast<float *>(ws + prefix_bytes);
-  p.ws_m = p.ws_acc + slots * HD;
-  p.ws_l = p.ws_m + slots;
-  paged_decode_flat_kernel<T, HD><<<dim3((unsigned)wgs), 256, 0, stream>>>(p);
-  check_launch("paged_attention");
-  // Measurement aid: HIPATTN_DECODE_NO_REDUCE=1 leaves the merge of the partials out, so that events around a
-  // call time the streaming kernel alone (the output is then incomplete).
-  if (const char *e = getenv("HIPATTN_DECODE_NO_REDUCE")) {
-    if (atoi(e) != 0) return;
-  }
-  paged_decode_flat_reduce_kernel<T, HD><<<dim3((unsigned)p.Hq, (unsigned)S), HD <= 64 ? 64 : 128, 0, stream>>>(p);
-  check_launch("paged_attention reduce");
-}
-
-template <typename T>
-void dispatch_head_flat(const DecodeParams &p, int head_size, int64_t S, int max_context_len, hipStream_t stream) {
+int flat_resident_workgroups(int dtype, int head_size) {
+#define HA_RES(H) \
+  case H: return dtype == HIPATTN_F16 ? flat_resident_workgroups<half_t, H>() : flat_resident_workgroups<bf16_t, H>()
   switch (head_size) {
-    case 64: launch_decode_flat<T, 64>(p, S, max_context_len, stream); break;
-    case 80: launch_decode_flat<T, 80>(p, S, max_context_len, stream); break;
-    case 96: launch_decode_flat<T, 96>(p, S, max_context_len, stream); break;
-    case 112: launch_decode_flat<T, 112>(p, S, max_context_len, stream); break;
-    case 128: launch_decode_flat<T, 128>(p, S, max_context_len, stream); break;
-    case 256: launch_decode_flat<T, 256>(p, S, max_context_len, stream); break;
+    HA_RES(64);
+    HA_RES(80);
+    HA_RES(96);
+    HA_RES(112);
+    HA_RES(128);
+    HA_RES(256);
     default: fail("paged_attention: unsupported head size %d (supported: 64, 80, 96, 112, 128, 256)", head_size);
   }
+#undef HA_RES
 }
+
+// How a call is carried out and what scratch memory it needs: computed from the shapes alone, so that
+// hipattn_paged_attention_workspace_size and the launch agree.
+struct DecodePlan {
+  bool generic = false, flat = false;
+  int part_blocks = 0;  // partitioned launch: KV blocks per partition
+  int num_parts = 1;    // partitioned / generic launch
+  int flat_wgs = 0, flat_cols = 0;
+  size_t prefix_bytes = 0;  // flat: the block-pair prefix table at the start of the scratch memory
+  size_t slots = 0;          // partial results (each head_size + 2 floats)
+  size_t bytes = 0;          // scratch memory in all
+};
+
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 // v1 takes the flat split for long steps: measured on MI355X it wins a few
 // percent once every wavefront of the launch has tens of block pairs to
 // stream, and loses to the partitioned launch (whose many short workgroups
 // hide the per-segment load chains behind each other) on short contexts or
 // small batches.  Its bookkeeping also needs the sequence table to fit in LDS
-// and unit indices in 32 bits.  HIPATTN_DECODE_FLAT=0/1 forces the choice
-// (tuning aid).
+// and unit indices in 32 bits.  The tuning switch decode_flat forces the choice.
 bool use_flat_split(int64_t S, int hk, int max_context_len) {
   if (S > kFlatMaxSeqs || max_context_len <= 0) return false;
   const int64_t max_units = S * hk * ((max_context_len + 2 * kBlockSize - 1) / (2 * kBlockSize));
   if (max_units >= (int64_t)1 << 30) return false;
-  if (const char *e = getenv("HIPATTN_DECODE_FLAT")) return atoi(e) != 0;
+  if (tuning().decode_flat >= 0) return tuning().decode_flat != 0;
   return max_context_len >= 1024 && max_units >= 32 * 2048;
 }
 
@@ -835,12 +824,10 @@ bool use_flat_split(int64_t S, int hk, int max_context_len) {
 // as the launch still has a couple of thousand workgroups (fewer fp32
 // partials, fewer start-up bubbles per byte); short contexts or small batches
 // get shorter partitions so that all CUs have work, never below 8 blocks.
-// HIPATTN_DECODE_PART_BLOCKS overrides the choice (tuning aid).
+// The tuning switch decode_part_blocks overrides the choice.
 int choose_part_blocks(int64_t S, int Hkv, int col_groups, int max_ctx) {
-  if (const char *e = getenv("HIPATTN_DECODE_PART_BLOCKS")) {
-    int v = atoi(e);
-    if (v >= 2 && v <= 64) return v + (v & 1);
-  }
+  const int forced = tuning().decode_part_blocks;
+  if (forced >= 2 && forced <= 64) return forced + (forced & 1);
   const int64_t max_blocks = (max_ctx + kBlockSize - 1) / kBlockSize;
   const int64_t items = S * Hkv * col_groups;  // workgroups per partition index
   const int64_t want_wgs = 2048;
@@ -851,6 +838,93 @@ int choose_part_blocks(int64_t S, int Hkv, int col_groups, int max_ctx) {
   if (pb < 8) pb = 8;
   if (pb > 64) pb = 64;
   return (int)pb;
+}
+
+DecodePlan plan_decode(int64_t S, int Hq, int Hkv, int head_size, int block_size, int dtype, int max_context_len) {
+  DecodePlan pl;
+  pl.generic = block_size != kBlockSize || dtype == HIPATTN_F32;
+  if (S <= 0 || Hq <= 0) return pl;
+  if (pl.generic) {
+    int64_t P = ((int64_t)max_context_len + kGenericPartTokens - 1) / kGenericPartTokens;
+    if (P < 1) P = 1;
+    HA_CHECK(P <= 65535, "paged_attention: max_context_len %d is too long", max_context_len);
+    pl.num_parts = (int)P;
+    if (P > 1) pl.slots = (size_t)S * Hq * P;
+  } else {
+    const int G = Hq / Hkv, col_groups = (G + 15) / 16;
+    pl.flat = use_flat_split(S, Hkv * col_groups, max_context_len);
+    if (pl.flat) {
+      const int64_t max_units = S * Hkv * col_groups * ((max_context_len + 2 * kBlockSize - 1) / (2 * kBlockSize));
+      // What the device holds at once, but no more than gives every wavefront two units of the largest
+      // possible step.
+      int64_t wgs = tuning().decode_flat_wgs > 0 ? tuning().decode_flat_wgs : flat_resident_workgroups(dtype, head_size);
+      const int64_t cap = (max_units + 7) / 8;
+      if (wgs > cap) wgs = cap;
+      pl.flat_wgs = (int)(wgs < 1 ? 1 : wgs);
+      pl.flat_cols = G < 16 ? G : 16;
+      pl.slots = (size_t)2 * pl.flat_wgs * 4 * pl.flat_cols;
+      pl.prefix_bytes = align256(((size_t)S + 1) * sizeof(int));
+    } else {
+      pl.part_blocks = choose_part_blocks(S, Hkv, col_groups, max_context_len);
+      const int64_t max_blocks = ((int64_t)max_context_len + kBlockSize - 1) / kBlockSize;
+      int64_t P = (max_blocks + pl.part_blocks - 1) / pl.part_blocks;
+      if (P < 1) P = 1;
+      pl.num_parts = (int)P;
+      if (P > 1) pl.slots = (size_t)S * Hq * P;
+    }
+  }
+  pl.bytes = pl.prefix_bytes + pl.slots * (size_t)(head_size + 2) * sizeof(float);
+  return pl;
+}
+
+// Where a call's scratch memory comes from.
+struct Scratch {
+  enum Kind { LIBRARY, CALLER } kind = LIBRARY;
+  void *ptr = nullptr;  // CALLER
+  int64_t bytes = 0;    // CALLER
+};
+
+// The scratch memory of one call (pl.bytes of it; nothing in it outlives the call).
+char *scratch_memory(const Scratch &from, const DecodePlan &pl, hipStream_t stream, const char *op) {
+  if (pl.bytes == 0) return nullptr;
+  switch (from.kind) {
+    case Scratch::CALLER:
+      HA_CHECK(from.ptr != nullptr, "%s: workspace is NULL but %zu bytes are needed", op, pl.bytes);
+      HA_CHECK((reinterpret_cast<uintptr_t>(from.ptr) & 255) == 0, "%s: workspace must be 256-byte aligned", op);
+      HA_CHECK(from.bytes >= 0 && (size_t)from.bytes >= pl.bytes,
+               "%s: workspace of %lld bytes is too small, %zu are needed (hipattn_paged_attention_workspace_size)", op,
+               (long long)from.bytes, pl.bytes);
+      return static_cast<char *>(from.ptr);
+    default:
+      return static_cast<char *>(library_workspace(WS_PAGED_ATTENTION, pl.bytes, stream));
+  }
+}
+
+template <typename T, int HD>
+void launch_decode_flat(DecodeParams p, const DecodePlan &pl, char *ws, hipStream_t stream) {
+  p.flat_waves = pl.flat_wgs * 4;
+  p.flat_cols = pl.flat_cols;
+  p.flat_prefix = reinterpret_cast<int *>(ws);
+  p.ws_acc = reinterpret_cast<float *>(ws + pl.prefix_bytes);
+  p.ws_m = p.ws_acc + pl.slots * HD;
+  p.ws_l = p.ws_m + pl.slots;
+  paged_decode_flat_kernel<T, HD><<<dim3((unsigned)pl.flat_wgs), 256, 0, stream>>>(p);
+  check_launch("paged_attention");
+  paged_decode_flat_reduce_kernel<T, HD><<<dim3((unsigned)p.Hq, (unsigned)p.num_seqs), HD <= 64 ? 64 : 128, 0, stream>>>(p);
+  check_launch("paged_attention reduce");
+}
+
+template <typename T>
+void dispatch_head_flat(const DecodeParams &p, int head_size, const DecodePlan &pl, char *ws, hipStream_t stream) {
+  switch (head_size) {
+    case 64: launch_decode_flat<T, 64>(p, pl, ws, stream); break;
+    case 80: launch_decode_flat<T, 80>(p, pl, ws, stream); break;
+    case 96: launch_decode_flat<T, 96>(p, pl, ws, stream); break;
+    case 112: launch_decode_flat<T, 112>(p, pl, ws, stream); break;
+    case 128: launch_decode_flat<T, 128>(p, pl, ws, stream); break;
+    case 256: launch_decode_flat<T, 256>(p, pl, ws, stream); break;
+    default: fail("paged_attention: unsupported head size %d (supported: 64, 80, 96, 112, 128, 256)", head_size);
+  }
 }
 
 GenericDecodeParams generic_params(const DecodeParams &p, int head_size, int block_size, float scale) {
@@ -876,6 +950,7 @@ GenericDecodeParams generic_params(const DecodeParams &p, int head_size, int blo
   g.head_size = head_size;
   g.block_size = block_size;
   g.num_seqs = p.num_seqs;
+  g.max_ctx = p.max_ctx;
   g.out = p.out;
   g.out_stride = p.out_stride;
   return g;
@@ -885,8 +960,8 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
                           hipattn_tensor *tmp_out, const hipattn_tensor *query, const hipattn_tensor *key_cache,
                           const hipattn_tensor *value_cache, int num_kv_heads, float scale,
                           const hipattn_tensor *block_tables, const hipattn_tensor *context_lens, int block_size,
-                          int max_context_len, const hipattn_tensor *alibi, bool v2, void *stream_arg) {
-  const char *op = v2 ? "paged_attention_v2" : "paged_attention_v1";
+                          int max_context_len, const hipattn_tensor *alibi, bool v2, const Scratch &scratch_from,
+                          const char *op, void *stream_arg) {
   check_tensor(out, "out", 3);
   check_tensor(query, "query", 3);
   check_tensor(key_cache, "key_cache", 5);
@@ -984,6 +1059,9 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
   p.num_seqs = (int)S;
   p.out = out->data;
   p.out_stride = out->strides[0];
+  // A context length beyond max_context_len (which sized the launch and the scratch memory) or beyond
+  // what a table row describes is cut there, in every kernel alike.
+  p.max_ctx = (int)std::min<int64_t>(max_context_len, block_tables->sizes[1] * block_size);
   const int64_t max_blocks = (max_context_len + block_size - 1) / block_size;
   if (v2) {
     check_tensor(exp_sums, "exp_sums", 3);
@@ -1010,7 +1088,7 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
       g.ws_l = static_cast<float *>(exp_sums->data);
       g.ws_m = static_cast<float *>(max_logits->data);
       g.tmp_out = tmp_out->data;
-      paged_decode_generic(g, query->dtype, true, max_context_len, stream);
+      paged_decode_generic(g, query->dtype, true, max_context_len, (int)P, nullptr, stream);
       return;
     }
     int64_t pb = (max_blocks + P - 1) / P;
@@ -1023,27 +1101,27 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
     p.ws_l = static_cast<float *>(exp_sums->data);
     p.ws_m = static_cast<float *>(max_logits->data);
     p.tmp_out = tmp_out->data;
-  } else if (generic) {
-    paged_decode_generic(generic_params(p, hd, block_size, scale), query->dtype, false, max_context_len, stream);
-    return;
-  } else if (use_flat_split(S, p.Hkv * p.col_groups, max_context_len)) {
-    if (query->dtype == HIPATTN_F16)
-      dispatch_head_flat<half_t>(p, hd, S, max_context_len, stream);
-    else
-      dispatch_head_flat<bf16_t>(p, hd, S, max_context_len, stream);
-    return;
   } else {
-    p.part_blocks = choose_part_blocks(S, p.Hkv, p.col_groups, max_context_len);
-    int64_t P = (max_blocks + p.part_blocks - 1) / p.part_blocks;
-    if (P < 1) P = 1;
-    p.num_parts = (int)P;
-    if (P > 1) {
-      const size_t n = (size_t)S * Hq * P;
-      const size_t acc_bytes = n * hd * sizeof(float);
-      char *ws = static_cast<char *>(library_workspace(acc_bytes + 2 * n * sizeof(float), stream));
+    const DecodePlan pl = plan_decode(S, Hq, num_kv_heads, hd, block_size, query->dtype, max_context_len);
+    char *ws = scratch_memory(scratch_from, pl, stream, op);
+    if (pl.generic) {
+      paged_decode_generic(generic_params(p, hd, block_size, scale), query->dtype, false, max_context_len, pl.num_parts,
+                           reinterpret_cast<float *>(ws), stream);
+      return;
+    }
+    if (pl.flat) {
+      if (query->dtype == HIPATTN_F16)
+        dispatch_head_flat<half_t>(p, hd, pl, ws, stream);
+      else
+        dispatch_head_flat<bf16_t>(p, hd, pl, ws, stream);
+      return;
+    }
+    p.part_blocks = pl.part_blocks;
+    p.num_parts = pl.num_parts;
+    if (pl.num_parts > 1) {
       p.ws_acc = reinterpret_cast<float *>(ws);
-      p.ws_m = reinterpret_cast<float *>(ws + acc_bytes);
-      p.ws_l = p.ws_m + n;
+      p.ws_m = p.ws_acc + pl.slots * hd;
+      p.ws_l = p.ws_m + pl.slots;
     }
   }
 #define HA_PA(TT)                                          \
@@ -1068,7 +1146,40 @@ extern "C" char *hipattn_paged_attention_v1(hipattn_tensor *out, const hipattn_t
                                             const hipattn_tensor *context_lens, int block_size, int max_context_len,
                                             const hipattn_tensor *alibi_slopes, void *stream) {
   HA_PROTECT(paged_attention_impl(out, nullptr, nullptr, nullptr, query, key_cache, value_cache, num_kv_heads, scale,
-                                  block_tables, context_lens, block_size, max_context_len, alibi_slopes, false, stream));
+                                  block_tables, context_lens, block_size, max_context_len, alibi_slopes, false, Scratch(),
+                                  "paged_attention_v1", stream));
+}
+
+extern "C" char *hipattn_paged_attention_v1_ws(hipattn_tensor *out, const hipattn_tensor *query,
+                                               const hipattn_tensor *key_cache, const hipattn_tensor *value_cache,
+                                               int num_kv_heads, float scale, const hipattn_tensor *block_tables,
+                                               const hipattn_tensor *context_lens, int block_size, int max_context_len,
+                                               const hipattn_tensor *alibi_slopes, void *workspace,
+                                               int64_t workspace_bytes, void *stream) {
+  HA_PROTECT({
+    Scratch from;
+    from.kind = Scratch::CALLER;
+    from.ptr = workspace;
+    from.bytes = workspace_bytes;
+    paged_attention_impl(out, nullptr, nullptr, nullptr, query, key_cache, value_cache, num_kv_heads, scale, block_tables,
+                         context_lens, block_size, max_context_len, alibi_slopes, false, from, "paged_attention_v1_ws",
+                         stream);
+  });
+}
+
+extern "C" char *hipattn_paged_attention_workspace_size(int64_t num_seqs, int num_heads, int num_kv_heads, int head_size,
+                                                        int block_size, int max_context_len, int32_t dtype,
+                                                        int64_t *bytes) {
+  HA_PROTECT({
+    HA_CHECK(bytes != nullptr, "paged_attention_workspace_size: bytes is NULL");
+    HA_CHECK(num_seqs >= 0 && num_heads >= 0 && max_context_len >= 0, "paged_attention_workspace_size: negative size");
+    HA_CHECK(is_float_dtype(dtype), "paged_attention_workspace_size: unsupported data type %s", dtype_name(dtype));
+    HA_CHECK(block_size == 8 || block_size == 16 || block_size == 32,
+             "paged_attention_workspace_size: unsupported block size %d (supported: 8, 16, 32)", block_size);
+    HA_CHECK(num_kv_heads > 0 && num_heads % num_kv_heads == 0,
+             "paged_attention_workspace_size: %d query heads not divisible by %d kv heads", num_heads, num_kv_heads);
+    *bytes = (int64_t)plan_decode(num_seqs, num_heads, num_kv_heads, head_size, block_size, dtype, max_context_len).bytes;
+  });
 }
 
 extern "C" char *hipattn_paged_attention_v2(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn_tensor *max_logits,
@@ -1078,5 +1189,6 @@ extern "C" char *hipattn_paged_attention_v2(hipattn_tensor *out, hipattn_tensor 
                                             const hipattn_tensor *context_lens, int block_size, int max_context_len,
                                             const hipattn_tensor *alibi_slopes, void *stream) {
   HA_PROTECT(paged_attention_impl(out, exp_sums, max_logits, tmp_out, query, key_cache, value_cache, num_kv_heads, scale,
-                                  block_tables, context_lens, block_size, max_context_len, alibi_slopes, true, stream));
+                                  block_tables, context_lens, block_size, max_context_len, alibi_slopes, true, Scratch(),
+                                  "paged_attention_v2", stream));
 }

@@ -24,6 +24,7 @@ struct GenericDecodeParams {
   int Hq, G;  // G = Hq / Hkv
   int head_size, block_size;
   int num_seqs;
+  int max_ctx;      // context lengths are clamped to this
   int part_tokens;  // tokens per partition, a multiple of block_size (set by paged_decode_generic)
   int num_parts;    // v2: given by the workspaces; v1: set by paged_decode_generic
   float *ws_acc;    // v1 partials [S, Hq, P, d] fp32
@@ -34,7 +35,13 @@ struct GenericDecodeParams {
   int64_t out_stride;
 };
 
-// Launches on `stream`; v1 takes its partials from the library workspace.
-void paged_decode_generic(GenericDecodeParams p, int dtype, bool v2, int max_context_len, hipStream_t stream);
+// Tokens per partition of the v1 launch.
+constexpr int kGenericPartTokens = 512;
+
+// Launches on `stream`.  v2: the workspaces of `p` give the partition count.  v1: `num_parts` partitions of
+// kGenericPartTokens tokens; with more than one, `scratch` holds num_seqs * Hq * num_parts * (head_size + 2)
+// floats for the partials.
+void paged_decode_generic(GenericDecodeParams p, int dtype, bool v2, int max_context_len, int num_parts, float *scratch,
+                          hipStream_t stream);
 
 }  // namespace hipattn

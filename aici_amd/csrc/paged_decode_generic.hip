@@ -14,7 +14,6 @@
 #include "common.h"
 #include "device_types.h"
 #include "paged_decode_generic.h"
-#include "workspace.h"
 
 namespace hipattn {
 
@@ -65,8 +64,7 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(GenericDecode
   const int qh = blockIdx.x, seq = blockIdx.y, part = blockIdx.z;
   const int tid = threadIdx.x;
   const int hd = p.head_size;
-  // a context cannot be longer than its table row can describe
-  const int ctx = min(p.context_lens[seq], p.table_cols * BS);
+  const int ctx = min(p.context_lens[seq], p.max_ctx);
   const int t0 = part * p.part_tokens;
   T *op = static_cast<T *>(p.out) + seq * p.out_stride + (int64_t)qh * hd;
   if (t0 >= ctx) {
@@ -111,7 +109,9 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(GenericDecode
     l += e;
   }
   l = wg_reduce(l, red, false);
-  const float inv = 1.0f / (l + 1e-6f);
+  // n >= 1 here and the largest term is exp(0), so l >= 1: the reference's guard against an empty sum
+  // (1 / (l + 1e-6), attention_kernels.cu:262) is not needed, and the MFMA kernels do without it too.
+  const float inv = 1.0f / l;
   for (int i = tid; i < n; i += 256) logits[i] = to_float(from_float<T>(logits[i] * inv));
   __syncthreads();
 
@@ -167,13 +167,13 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(GenericDecode
   }
 }
 
-// grid (Hq, S), 64 threads: out = sum_p o_p * l_p e^(m_p - M) / (sum_p l_p e^(m_p - M) + 1e-6).
+// grid (Hq, S), 64 threads: out = sum_p o_p * l_p e^(m_p - M) / sum_p l_p e^(m_p - M).
 template <typename T, bool V2FMT>
 __global__ __launch_bounds__(64) void paged_decode_generic_reduce_kernel(GenericDecodeParams p) {
   const int qh = blockIdx.x, seq = blockIdx.y;
   const int lane = threadIdx.x;
   const int hd = p.head_size;
-  const int ctx = min(p.context_lens[seq], p.table_cols * p.block_size);
+  const int ctx = min(p.context_lens[seq], p.max_ctx);
   if (ctx <= 0) return;  // the main kernel wrote the zero row
   const int np = (ctx + p.part_tokens - 1) / p.part_tokens;
   const int64_t base = ((int64_t)seq * p.Hq + qh) * p.num_parts;
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(64) void paged_decode_generic_reduce_kernel(Generic
   for (int i = lane; i < np; i += 64) denom += p.ws_l[base + i] * __expf(p.ws_m[base + i] - mmax);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) denom += __shfl_xor(denom, o, 64);
-  const float inv = 1.0f / (denom + 1e-6f);
+  const float inv = 1.0f / denom;  // ctx > 0: at least one partition with l >= 1 at the common maximum
   T *op = static_cast<T *>(p.out) + seq * p.out_stride + (int64_t)qh * hd;
   for (int d = lane; d < hd; d += 64) {
     float o = 0.f;
@@ -224,7 +224,8 @@ void dispatch_block(const GenericDecodeParams &p, hipStream_t stream) {
 
 }  // namespace
 
-void paged_decode_generic(GenericDecodeParams p, int dtype, bool v2, int max_context_len, hipStream_t stream) {
+void paged_decode_generic(GenericDecodeParams p, int dtype, bool v2, int max_context_len, int num_parts, float *scratch,
+                          hipStream_t stream) {
   const int x = 16 / dtype_size(dtype);
   HA_CHECK(p.head_size % x == 0 && p.head_size <= 256,
            "paged_attention: unsupported head size %d for block size %d / %s (a multiple of %d up to 256)", p.head_size,
@@ -239,17 +240,13 @@ void paged_decode_generic(GenericDecodeParams p, int dtype, bool v2, int max_con
     HA_CHECK(p.part_tokens <= 8192, "paged_attention_v2: %d partitions are too few for max_context_len %d (at most 8192 tokens each)",
              p.num_parts, max_context_len);
   } else {
-    p.part_tokens = 512;
-    int64_t P = ((int64_t)max_context_len + p.part_tokens - 1) / p.part_tokens;
-    if (P < 1) P = 1;
-    HA_CHECK(P <= 65535, "paged_attention: max_context_len %d is too long", max_context_len);
-    p.num_parts = (int)P;
-    if (P > 1) {
-      const size_t n = (size_t)p.num_seqs * p.Hq * P;
-      const size_t acc_bytes = n * p.head_size * sizeof(float);
-      char *ws = static_cast<char *>(library_workspace(acc_bytes + 2 * n * sizeof(float), stream));
-      p.ws_acc = reinterpret_cast<float *>(ws);
-      p.ws_m = reinterpret_cast<float *>(ws + acc_bytes);
+    p.part_tokens = kGenericPartTokens;
+    p.num_parts = num_parts;
+    if (num_parts > 1) {
+      HA_CHECK(scratch != nullptr, "paged_attention: no scratch memory for %d partitions", num_parts);
+      const size_t n = (size_t)p.num_seqs * p.Hq * num_parts;
+      p.ws_acc = scratch;
+      p.ws_m = scratch + n * p.head_size;
       p.ws_l = p.ws_m + n;
     }
   }

@@ -45,6 +45,12 @@
 
 #include "common.h"
 #include "device_types.h"
+#include "workspace.h"
+
+// The global -> LDS copies below set M0 inside inline asm and say so in their clobber lists, so that the
+// compiler never assumes a value of its own survives them.  M0 is a register the compiler reserves, and
+// naming a reserved register there draws a warning per use; the declaration is wanted all the same.
+#pragma clang diagnostic ignored "-Winline-asm"
 
 // Phase timeline of one workgroup of the eight-wavefront kernel: built with
 // -DHIPATTN_PHASE_TRACE=<workgroup id>, lane 0 of every wavefront of that
@@ -664,7 +670,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:" #OFF \
                :                                                                                   \
                : "s"(dst), "v"(dma_lane), "s"(src)                                                 \
-               : "memory")
+               : "memory", "m0")
     switch (i) {
       case 0: HA_DMA_PIECE(0); break;
       case 1: HA_DMA_PIECE(1024); break;
@@ -1122,16 +1128,16 @@ void pick_qt(const PrefillParams &p, int64_t total_q, hipStream_t stream) {
   // 128-token sequence: 17 us either way -- so the four-wavefront kernel is left with what the other does not
   // do: head sizes above 128, sliding windows, rows too far apart for 32-bit offsets.
   if constexpr (HDP <= 128) {
-    const char *force = getenv("HIPATTN_PREFILL_KERNEL");  // tuning aid: "w8", "qt2" or "qt1"
+    const int force = tuning().prefill_kernel;  // 0: choose here; 1: eight wavefronts; 2 / 3: four wavefronts, 2 / 1 row tiles
     // the eight-wavefront kernel addresses a tile's 64 rows with 32-bit byte offsets
     const bool fits = p.k_row < (1 << 23) && p.v_row < (1 << 23);
     // it knows the causal mask and no mask; other windows go to the four-wavefront kernel
     const bool plain = p.win_left < 0 && p.win_right <= 0;
-    if (plain && fits && (force ? !strcmp(force, "w8") : true)) {
+    if (plain && fits && (force == 0 || force == 1)) {
       launch_prefill_w8<T, HDP>(p, stream);
       return;
     }
-    if (force ? !strcmp(force, "qt2") : false) {
+    if (force == 2) {
       launch_prefill<T, HDP, 2>(p, stream);
       return;
     }
@@ -1279,9 +1285,8 @@ template <typename T>
 void dispatch_paged(const PrefillParams &p, hipStream_t stream) {
   const int hdp = ((p.d + 31) / 32) * 32;
   // Head sizes that fill their MFMA tiles take the block images as they are (16-byte aligned images); the
-  // others are staged through registers, which pads them.  HIPATTN_PAGED_PREFILL_DMA=0 forces the staged form (tuning aid).
-  const char *force = getenv("HIPATTN_PAGED_PREFILL_DMA");
-  const bool dma = p.d == hdp && p.vc_block % 8 == 0 && p.vc_head % 8 == 0 && !(force && force[0] == '0');
+  // others are staged through registers, which pads them.  The tuning switch paged_prefill_dma = 0 forces the staged form.
+  const bool dma = p.d == hdp && p.vc_block % 8 == 0 && p.vc_head % 8 == 0 && tuning().paged_prefill_dma != 0;
 #define HA_W8P(H)                                              \
   if (dma) launch_prefill_w8<T, H, W8_PAGED_DMA>(p, stream);   \
   else launch_prefill_w8<T, H, W8_PAGED>(p, stream)

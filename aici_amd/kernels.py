@@ -103,6 +103,39 @@ def paged_attention_v1(out: torch.Tensor, query: torch.Tensor, key_cache: torch.
          _stream(query))
 
 
+def paged_attention_workspace_size(num_seqs: int, num_heads: int, num_kv_heads: int, head_size: int, block_size: int,
+                                   max_context_len: int, dtype: torch.dtype) -> int:
+    """Bytes of scratch memory paged_attention_v1 needs for these shapes on the current device."""
+    n = ctypes.c_int64(0)
+    call("hipattn_paged_attention_workspace_size", int(num_seqs), int(num_heads), int(num_kv_heads), int(head_size),
+         int(block_size), int(max_context_len), _DTYPES[dtype], ctypes.byref(n))
+    return int(n.value)
+
+
+def paged_attention_v1_ws(out: torch.Tensor, query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                          num_kv_heads: int, scale: float, block_tables: torch.Tensor, context_lens: torch.Tensor,
+                          block_size: int, max_context_len: int, workspace: Optional[torch.Tensor],
+                          alibi_slopes: Optional[torch.Tensor] = None) -> None:
+    """paged_attention_v1 on a caller-provided scratch tensor (uint8, on the GPU; None when none is needed)."""
+    ptr = ctypes.c_void_p(workspace.data_ptr()) if workspace is not None else None
+    nbytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    call("hipattn_paged_attention_v1_ws", _desc(out, "out"), _desc(query, "query"), _desc(key_cache, "key_cache"),
+         _desc(value_cache, "value_cache"), int(num_kv_heads), float(scale), _desc(block_tables, "block_tables"),
+         _desc(context_lens, "context_lens"), int(block_size), int(max_context_len), _desc(alibi_slopes, "alibi"),
+         ptr, int(nbytes), _stream(query))
+
+
+def tuning_set(name: str, value: int) -> None:
+    """Sets one of the library's tuning switches (see hipattn_tuning_set in hipattn.h)."""
+    call("hipattn_tuning_set", name.encode(), int(value))
+
+
+def tuning_get(name: str) -> int:
+    v = ctypes.c_int(0)
+    call("hipattn_tuning_get", name.encode(), ctypes.byref(v))
+    return int(v.value)
+
+
 def paged_attention_v2(out: torch.Tensor, exp_sums: torch.Tensor, max_logits: torch.Tensor, tmp_out: torch.Tensor,
                        query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, num_kv_heads: int,
                        scale: float, block_tables: torch.Tensor, context_lens: torch.Tensor, block_size: int,

@@ -109,8 +109,13 @@ char *hipattn_mha_varlen_fwd_paged(const hipattn_tensor *q, const hipattn_tensor
 /* Replaces paged_attention_v1_C (lib.rs:107-120; attention_kernels.cu:679-700).
  * out/query [S, Hq, d]; key_cache [nb, Hkv, d/x, BS, x]; value_cache
  * [nb, Hkv, d, BS]; block_tables int32 [S, max_blocks]; context_lens int32 [S].
- * alibi_slopes f32 [Hq] or NULL.  Runs the split-K kernel on a workspace the
- * library owns (grown with hipMalloc when a call needs more than it has).
+ * alibi_slopes f32 [Hq] or NULL.  A context length above max_context_len is
+ * cut there.  Runs the split-K kernels on scratch memory the library owns: one
+ * buffer per (device, stream), so calls on different streams may overlap; it
+ * grows with hipMalloc when a call needs more than it has (the old buffer stays
+ * alive until hipattn_shutdown, nothing is synchronised); a stream that is being
+ * captured into a graph cannot grow it -- run the call once with the largest
+ * shapes before capturing, or use hipattn_paged_attention_v1_ws.
  * x = 16 / sizeof(dtype).  The reference's support matrix is accepted: f16,
  * bf16 and f32; BS 8, 16 and 32; d in {64, 80, 96, 112, 128, 256}.  BS = 16 in
  * a 2-byte type (what rLLM runs) takes the MFMA kernels; the other
@@ -126,6 +131,35 @@ char *hipattn_paged_attention_v1(hipattn_tensor *out,
                                  int block_size, int max_context_len,
                                  const hipattn_tensor *alibi_slopes,
                                  void *stream);
+
+/* hipattn_paged_attention_v1 on scratch memory the caller provides: the
+ * "workspace-size query + caller-allocated split-K scratch" form of the call
+ * (the reference's v1 signature has no such argument, lib.rs:107-120; its v2
+ * passes three tensors).  workspace: device memory, 256-byte aligned, of at
+ * least the number of bytes hipattn_paged_attention_workspace_size reports for
+ * these shapes (NULL is fine when that is 0); its contents need not be
+ * preserved or cleared between calls.  Calls that overlap in time need
+ * workspaces of their own. */
+char *hipattn_paged_attention_v1_ws(hipattn_tensor *out,
+                                    const hipattn_tensor *query,
+                                    const hipattn_tensor *key_cache,
+                                    const hipattn_tensor *value_cache,
+                                    int num_kv_heads, float scale,
+                                    const hipattn_tensor *block_tables,
+                                    const hipattn_tensor *context_lens,
+                                    int block_size, int max_context_len,
+                                    const hipattn_tensor *alibi_slopes,
+                                    void *workspace, int64_t workspace_bytes,
+                                    void *stream);
+
+/* Scratch bytes hipattn_paged_attention_v1* needs on the current device for
+ * num_seqs sequences of at most max_context_len tokens (0 when the call needs
+ * none).  Depends on the shapes only, not on the context lengths of a step. */
+char *hipattn_paged_attention_workspace_size(int64_t num_seqs, int num_heads,
+                                             int num_kv_heads, int head_size,
+                                             int block_size,
+                                             int max_context_len, int32_t dtype,
+                                             int64_t *bytes);
 
 /* Replaces paged_attention_v2_C (lib.rs:122-137; attention_kernels.cu:421-546,
  * 729-874).  Same as v1 with caller-provided split-K workspaces: exp_sums and
@@ -281,7 +315,7 @@ typedef struct hipattn_device_props {
  * hipMemGetInfo: current = total - free on the device, peak = the largest
  * `current` seen by any stats call since the last reset. */
 char *hipattn_reset_peak_memory_stats(int device);
-char *hipattn_empty_cache(void);
+char *hipattn_empty_cache(void); /* nothing to release: no caching allocator; see hipattn_shutdown */
 char *hipattn_get_stats_allocated_bytes(int device, hipattn_mem_stats *outp);
 char *hipattn_get_device_properties(int device, hipattn_device_props *outp);
 
@@ -325,8 +359,23 @@ char *hipattn_event_query(hipattn_event *e, int *done);
 char *hipattn_event_synchronize(hipattn_event *e);
 char *hipattn_event_free(hipattn_event *e);
 
-/* Releases the library-owned split-K workspace of every device. */
+/* Releases the scratch buffers the library owns, on every device, after
+ * waiting for the devices to drain.  Graphs captured from calls that used them
+ * must not be replayed afterwards. */
 char *hipattn_shutdown(void);
+
+/* Switches for tuning and for tests that want one particular kernel.  Each is
+ * read from the environment once, when the library is loaded (HIPATTN_ + the
+ * name in capitals); ops never read the environment.  Names: decode_flat
+ * (-1 library's choice, 0 partitioned launch, 1 flat split), decode_flat_wgs
+ * (0 = what the device holds at once), decode_part_blocks (0 = chosen per
+ * call, else 2..64), prefill_kernel (0 library's choice, 1 eight wavefronts,
+ * 2 / 3 four wavefronts with 2 / 1 row tiles), paged_prefill_dma (-1 library's
+ * choice, 0 staged tiles), cache_move_lds (-1 library's choice, 0 never the
+ * LDS-transposing kernels).  Every setting computes the same results.  Not
+ * synchronised with running calls: set them between calls. */
+char *hipattn_tuning_set(const char *name, int value);
+char *hipattn_tuning_get(const char *name, int *value);
 
 /* ---------------------------------------------------------------------------
  * Host side of the paged KV cache (no GPU needed)

@@ -15,8 +15,8 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("decode_launch", ["flat", "partitioned"])
-def test_captured_step_replays_like_eager(device, monkeypatch, decode_launch):
-    monkeypatch.setenv("HIPATTN_DECODE_FLAT", "1" if decode_launch == "flat" else "0")
+def test_captured_step_replays_like_eager(device, tuning, decode_launch):
+    tuning("decode_flat", 1 if decode_launch == "flat" else 0)
     dtype, Hq, Hkv, d, bs = torch.bfloat16, 32, 8, 128, 16
     g = torch.Generator().manual_seed(51)
     # prefill rows: 3 sequences with some prior context; decode rows: 40 sequences and 3
@@ -83,11 +83,13 @@ def test_captured_step_replays_like_eager(device, monkeypatch, decode_launch):
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         fill(1)
-        step()      # grows the library's workspace and sets kernel attributes outside the capture
+        step()      # grows the library's scratch buffers of this stream and sets kernel attributes outside the capture
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    # captured on the stream that was warmed up: the library keeps its scratch buffers per stream and
+    # cannot grow one during a capture
+    with torch.cuda.graph(graph, stream=side):
         graph_outs = step()
     kc0, vc0 = kc.clone(), vc.clone()
     for seed in (2, 3, 4):

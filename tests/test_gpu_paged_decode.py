@@ -15,14 +15,11 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.fixture(autouse=True, params=["auto", "flat", "partitioned"])
-def launch_strategy(request, monkeypatch):
+def launch_strategy(request, tuning):
     """paged_attention_v1 has two launch strategies (one list of block pairs cut into equal
     ranges per wavefront, or one workgroup per context partition) and picks by problem size;
     every test runs under the library's own choice and with each one forced."""
-    if request.param == "auto":
-        monkeypatch.delenv("HIPATTN_DECODE_FLAT", raising=False)
-    else:
-        monkeypatch.setenv("HIPATTN_DECODE_FLAT", "1" if request.param == "flat" else "0")
+    tuning("decode_flat", {"auto": -1, "flat": 1, "partitioned": 0}[request.param])
     return request.param
 
 
@@ -280,4 +277,93 @@ def test_other_block_sizes_edges_alibi_and_stale_slots(device, dtype, bs):
     assert not torch.isnan(out).any()
     assert torch.all(out[0] == 0)   # no context: a zero row, as the oracle gives
     tol = 5e-5 if dtype == torch.float32 else TOL[dtype]
+    assert (out.cpu().float() - want).abs().max().item() <= tol
+
+
+# ---- scratch memory: caller-provided workspaces, streams, context lengths beyond the stated maximum ----
+
+WS_CASES = [
+    ("flat", (40, 900, 2048, 32, 8, 128, torch.bfloat16, 4000)),
+    ("partitioned", (9, 1, 1500, 32, 8, 128, torch.float16, 1024)),
+    ("flat_wide_groups", (24, 1000, 3000, 40, 1, 128, torch.bfloat16, 4800)),
+]
+
+
+@pytest.mark.parametrize("name,shape", WS_CASES, ids=[n for n, _ in WS_CASES])
+def test_caller_workspace_entry_matches_v1(device, name, shape):
+    """hipattn_paged_attention_v1_ws on a workspace of exactly the reported size, filled with
+    garbage (nothing in it has to survive or be prepared between calls): bit-identical to v1, twice in a
+    row on the same workspace, and no byte outside the reported size is touched."""
+    S, lo, hi, Hq, Hkv, d, dtype, pool = shape
+    c = W.decode_inputs(41, S, lo, hi, Hq, Hkv, d, dtype, pool)
+    dd = c.to(device)
+    want = torch.full_like(dd.q, float("nan"))
+    K.paged_attention_v1(want, dd.q, dd.key_cache, dd.value_cache, Hkv, c.scale, dd.block_tables, dd.context_lens,
+                         16, c.max_ctx)
+    n = K.paged_attention_workspace_size(S, Hq, Hkv, d, 16, c.max_ctx, dtype)
+    assert n >= 0 and n % 4 == 0
+    guard = 4096
+    ws = torch.full((n + guard,), 0xA5, dtype=torch.uint8, device=device)
+    for _ in range(2):
+        out = torch.full_like(dd.q, float("nan"))
+        K.paged_attention_v1_ws(out, dd.q, dd.key_cache, dd.value_cache, Hkv, c.scale, dd.block_tables,
+                                dd.context_lens, 16, c.max_ctx, ws[:n] if n else None)
+        assert torch.equal(out, want)
+    assert torch.all(ws[n:] == 0xA5)
+    if n:
+        with pytest.raises(HipAttnError, match="too small"):
+            K.paged_attention_v1_ws(out, dd.q, dd.key_cache, dd.value_cache, Hkv, c.scale, dd.block_tables,
+                                    dd.context_lens, 16, c.max_ctx, ws[:n - 256])
+        with pytest.raises(HipAttnError, match="workspace is NULL"):
+            K.paged_attention_v1_ws(out, dd.q, dd.key_cache, dd.value_cache, Hkv, c.scale, dd.block_tables,
+                                    dd.context_lens, 16, c.max_ctx, None)
+    assert (want.cpu().float() - oracle(c)).abs().max().item() <= TOL[dtype]
+
+
+def test_two_streams_share_nothing(device):
+    """v1 keeps its scratch memory per stream: two streams running steps of different sizes at the
+    same time both get the results they get when run alone."""
+    a = W.decode_inputs(42, 48, 1000, 4096, 32, 8, 128, torch.bfloat16, 9000)
+    b = W.decode_inputs(43, 7, 200, 1400, 32, 8, 128, torch.bfloat16, 700)
+    da, db = a.to(device), b.to(device)
+
+    def call(d, c, out):
+        K.paged_attention_v1(out, d.q, d.key_cache, d.value_cache, 8, c.scale, d.block_tables, d.context_lens, 16,
+                             c.max_ctx)
+
+    alone_a, alone_b = torch.empty_like(da.q), torch.empty_like(db.q)
+    call(da, a, alone_a)
+    call(db, b, alone_b)
+    torch.cuda.synchronize()
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    outs_a = [torch.full_like(da.q, float("nan")) for _ in range(6)]
+    outs_b = [torch.full_like(db.q, float("nan")) for _ in range(6)]
+    for i in range(6):  # interleaved enqueues: the two streams' kernels overlap on the device
+        with torch.cuda.stream(sa):
+            call(da, a, outs_a[i])
+        with torch.cuda.stream(sb):
+            call(db, b, outs_b[i])
+    torch.cuda.synchronize()
+    for o in outs_a:
+        assert torch.equal(o, alone_a)
+    for o in outs_b:
+        assert torch.equal(o, alone_b)
+    assert (alone_a.cpu().float()[::6] - oracle(a, rows=list(range(0, 48, 6)))).abs().max().item() <= TOL[torch.bfloat16]
+    assert (alone_b.cpu().float() - oracle(b)).abs().max().item() <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("dtype,bs", [(torch.bfloat16, 16), (torch.float32, 16), (torch.float16, 8)])
+def test_context_lengths_above_the_stated_maximum_are_cut_there(device, dtype, bs):
+    """A context_lens entry above max_context_len: every kernel attends to the first max_context_len
+    tokens, as if the entry had been that."""
+    c = W.decode_inputs(44, 6, 300, 1200, 8, 2, 128, dtype, 6 * (1200 // bs + 1), block_size=bs)
+    cut = 640
+    dd = c.to(device)
+    out = torch.full_like(dd.q, float("nan"))
+    K.paged_attention_v1(out, dd.q, dd.key_cache, dd.value_cache, 2, c.scale, dd.block_tables, dd.context_lens, bs,
+                         cut)
+    want = ref.paged_attention(c.q.float(), c.key_cache.float(), c.value_cache.float(), 2, c.scale, c.block_tables,
+                               torch.clamp(c.context_lens, max=cut), bs)
+    tol = FP32_TOL if dtype == torch.float32 else TOL[dtype]
+    assert not torch.isnan(out).any()
     assert (out.cpu().float() - want).abs().max().item() <= tol

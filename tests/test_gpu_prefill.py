@@ -16,14 +16,11 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.fixture(autouse=True, params=["auto", "eight_wavefronts", "four_wavefronts"])
-def kernel_choice(request, monkeypatch):
+def kernel_choice(request, tuning):
     """The forward pass has two kernels (256-row workgroups of eight wavefronts for head sizes up to
     128, 128-row workgroups of four) and picks by launch size; every test runs under the library's
     own choice and with each one forced (head sizes above 128 always take the second)."""
-    if request.param == "auto":
-        monkeypatch.delenv("HIPATTN_PREFILL_KERNEL", raising=False)
-    else:
-        monkeypatch.setenv("HIPATTN_PREFILL_KERNEL", "w8" if request.param == "eight_wavefronts" else "qt1")
+    tuning("prefill_kernel", {"auto": 0, "eight_wavefronts": 1, "four_wavefronts": 3}[request.param])
     return request.param
 
 

@@ -18,14 +18,11 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.fixture(autouse=True, params=["auto", "staged"])
-def tile_route(request, monkeypatch):
+def tile_route(request, tuning):
     """Head sizes that fill their MFMA tiles (32, 64, 96, 128) have their tiles copied from the cache into
-    LDS as block images; the others -- and every size when HIPATTN_PAGED_PREFILL_DMA=0 -- are staged
+    LDS as block images; the others -- and every size when the tuning switch paged_prefill_dma is 0 -- are staged
     through registers.  Every test runs both ways."""
-    if request.param == "auto":
-        monkeypatch.delenv("HIPATTN_PAGED_PREFILL_DMA", raising=False)
-    else:
-        monkeypatch.setenv("HIPATTN_PAGED_PREFILL_DMA", "0")
+    tuning("paged_prefill_dma", -1 if request.param == "auto" else 0)
     return request.param
 
 
