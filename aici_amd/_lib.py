@@ -80,6 +80,8 @@ _ERR_FUNCS = {
     "hipattn_paged_attention_v1": [TP, TP, TP, TP, c_int, c_float, TP, TP, c_int, c_int, TP, c_void_p],
     "hipattn_paged_attention_v1_ws": [TP, TP, TP, TP, c_int, c_float, TP, TP, c_int, c_int, TP, c_void_p, c_int64,
                                       c_void_p],
+    "hipattn_paged_attention_v1_static": [TP, TP, TP, TP, c_int, c_float, TP, TP, c_int, c_int, TP, c_void_p],
+    "hipattn_init": [],
     "hipattn_paged_attention_workspace_size": [c_int64, c_int, c_int, c_int, c_int, c_int, c_int32, POINTER(c_int64)],
     "hipattn_paged_attention_v2": [TP, TP, TP, TP, TP, TP, TP, c_int, c_float, TP, TP, c_int, c_int, TP, c_void_p],
     "hipattn_reshape_and_cache": [TP, TP, TP, TP, TP, c_void_p],

@@ -879,10 +879,32 @@ DecodePlan plan_decode(int64_t S, int Hq, int Hkv, int head_size, int block_size
 
 // Where a call's scratch memory comes from.
 struct Scratch {
-  enum Kind { LIBRARY, CALLER } kind = LIBRARY;
+  enum Kind { LIBRARY, CALLER, STATIC } kind = LIBRARY;
   void *ptr = nullptr;  // CALLER
   int64_t bytes = 0;    // CALLER
 };
+
+// The scratch array of hipattn_paged_attention_v1_static, the entry point that allocates nothing: device
+// memory that exists from the moment the code object is loaded, one copy per device.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; kernels get the address that call returns.
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// The address of `scratch` on the current device, asked of the runtime once per device.
+char *static_scratch() {
+  constexpr int kDevices = 64;
+  static std::atomic<char *> address[kDevices];
+  int dev = 0;
+  HA_HIP(hipGetDevice(&dev));
+  HA_CHECK(dev >= 0 && dev < kDevices, "device index %d out of range", dev);
+  char *ptr = address[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    HA_HIP(hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)));
+    HA_CHECK(ptr != nullptr, "hipGetSymbolAddress returned no address for the scratch array");
+    address[dev].store(ptr, std::memory_order_release);
+  }
+  return ptr;
+}
 
 // The scratch memory of one call (pl.bytes of it; nothing in it outlives the call).
 char *scratch_memory(const Scratch &from, const DecodePlan &pl, hipStream_t stream, const char *op) {
@@ -895,6 +917,12 @@ char *scratch_memory(const Scratch &from, const DecodePlan &pl, hipStream_t stre
                "%s: workspace of %lld bytes is too small, %zu are needed (hipattn_paged_attention_workspace_size)", op,
                (long long)from.bytes, pl.bytes);
       return static_cast<char *>(from.ptr);
+    case Scratch::STATIC:
+      HA_CHECK(pl.bytes <= kStaticScratchBytes,
+               "%s: this call needs %zu bytes of scratch memory, more than the %zu bytes of the built-in array; use "
+               "hipattn_paged_attention_v1 or hipattn_paged_attention_v1_ws for it",
+               op, pl.bytes, kStaticScratchBytes);
+      return static_scratch();
     default:
       return static_cast<char *>(library_workspace(WS_PAGED_ATTENTION, pl.bytes, stream));
   }
@@ -1164,6 +1192,28 @@ extern "C" char *hipattn_paged_attention_v1_ws(hipattn_tensor *out, const hipatt
     paged_attention_impl(out, nullptr, nullptr, nullptr, query, key_cache, value_cache, num_kv_heads, scale, block_tables,
                          context_lens, block_size, max_context_len, alibi_slopes, false, from, "paged_attention_v1_ws",
                          stream);
+  });
+}
+
+extern "C" char *hipattn_paged_attention_v1_static(hipattn_tensor *out, const hipattn_tensor *query,
+                                                   const hipattn_tensor *key_cache, const hipattn_tensor *value_cache,
+                                                   int num_kv_heads, float scale, const hipattn_tensor *block_tables,
+                                                   const hipattn_tensor *context_lens, int block_size,
+                                                   int max_context_len, const hipattn_tensor *alibi_slopes, void *stream) {
+  HA_PROTECT({
+    Scratch from;
+    from.kind = Scratch::STATIC;
+    paged_attention_impl(out, nullptr, nullptr, nullptr, query, key_cache, value_cache, num_kv_heads, scale, block_tables,
+                         context_lens, block_size, max_context_len, alibi_slopes, false, from, "paged_attention_v1_static",
+                         stream);
+  });
+}
+
+extern "C" char *hipattn_init(void) {
+  HA_PROTECT({
+    (void)static_scratch();
+    for (int dtype : {HIPATTN_F16, HIPATTN_BF16})
+      for (int hd : {64, 80, 96, 112, 128, 256}) (void)flat_resident_workgroups(dtype, hd);
   });
 }
 

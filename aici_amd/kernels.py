@@ -125,6 +125,22 @@ def paged_attention_v1_ws(out: torch.Tensor, query: torch.Tensor, key_cache: tor
          ptr, int(nbytes), _stream(query))
 
 
+def paged_attention_v1_static(out: torch.Tensor, query: torch.Tensor, key_cache: torch.Tensor,
+                              value_cache: torch.Tensor, num_kv_heads: int, scale: float, block_tables: torch.Tensor,
+                              context_lens: torch.Tensor, block_size: int, max_context_len: int,
+                              alibi_slopes: Optional[torch.Tensor] = None) -> None:
+    """paged_attention_v1 on the library's built-in scratch array: allocates nothing."""
+    call("hipattn_paged_attention_v1_static", _desc(out, "out"), _desc(query, "query"), _desc(key_cache, "key_cache"),
+         _desc(value_cache, "value_cache"), int(num_kv_heads), float(scale), _desc(block_tables, "block_tables"),
+         _desc(context_lens, "context_lens"), int(block_size), int(max_context_len), _desc(alibi_slopes, "alibi"),
+         _stream(query))
+
+
+def init() -> None:
+    """Set-up for the current device ahead of the first call (hipattn_init)."""
+    call("hipattn_init")
+
+
 def tuning_set(name: str, value: int) -> None:
     """Sets one of the library's tuning switches (see hipattn_tuning_set in hipattn.h)."""
     call("hipattn_tuning_set", name.encode(), int(value))

@@ -152,6 +152,34 @@ char *hipattn_paged_attention_v1_ws(hipattn_tensor *out,
                                     void *workspace, int64_t workspace_bytes,
                                     void *stream);
 
+/* hipattn_paged_attention_v1 for callers that cannot allocate (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc); it has
+ * no counterpart in the reference.  Same arguments and results as
+ * hipattn_paged_attention_v1, but the split-K scratch memory is a 16 MiB array
+ * built into the library's code object (each device the library runs on holds
+ * it until the process ends), so the call allocates and frees nothing.  A call
+ * whose shapes need more (hipattn_paged_attention_workspace_size) is refused
+ * with a message.  Every call on a device uses that device's one array: calls
+ * that overlap in time on one device (two streams, two threads) race.  The
+ * first call on a device asks the runtime for the array's address and for the
+ * decode kernels' occupancy; hipattn_init does that ahead of time. */
+char *hipattn_paged_attention_v1_static(hipattn_tensor *out,
+                                        const hipattn_tensor *query,
+                                        const hipattn_tensor *key_cache,
+                                        const hipattn_tensor *value_cache,
+                                        int num_kv_heads, float scale,
+                                        const hipattn_tensor *block_tables,
+                                        const hipattn_tensor *context_lens,
+                                        int block_size, int max_context_len,
+                                        const hipattn_tensor *alibi_slopes,
+                                        void *stream);
+
+/* Optional set-up for the current device: everything the decode entry points
+ * would otherwise ask the runtime on their first call (the address of the
+ * built-in scratch array, kernel occupancy).  Allocates nothing; safe to call
+ * more than once. */
+char *hipattn_init(void);
+
 /* Scratch bytes hipattn_paged_attention_v1* needs on the current device for
  * num_seqs sequences of at most max_context_len tokens (0 when the call needs
  * none).  Depends on the shapes only, not on the context lengths of a step. */
