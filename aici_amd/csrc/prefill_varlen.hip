@@ -76,7 +76,6 @@ namespace {
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr int BN = 64;  // keys per LDS tile
-constexpr float kRescaleThreshold = 8.0f;  // log2 units: probabilities stay below 256
 
 struct PrefillParams {
   const void *q, *k, *v;
@@ -102,6 +101,10 @@ struct PrefillParams {
   int table_cols;
   int64_t num_blocks;
   int64_t kc_block, kc_head, vc_block, vc_head;  // cache strides in elements
+  // out holds fp32 instead of the input type: the accumulators divided by the row sums, not rounded again
+  // (for checking the kernel's arithmetic apart from the rounding of its output; o_row / o_head count floats).
+  int out_f32;
+  float rescale_thr;  // a row's reference maximum moves when the row outgrows it by more than this (log2 units)
 };
 
 template <typename T>
@@ -329,7 +332,7 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
 #pragma unroll
           for (int i = 1; i < 16; i++) mx = fmaxf(mx, s[qt][i]);
           mx = max_across_halves(mx) * p.scale_log2;
-          const bool grow = mx > m_run[qt] + kRescaleThreshold;
+          const bool grow = mx > m_run[qt] + p.rescale_thr;
           if (__builtin_expect(__any(grow), 0)) {
             const float m_new = grow ? mx : m_run[qt];
             // exp2(-inf - finite) = 0 on a row's first keys; rows that do not grow keep 1
@@ -398,6 +401,7 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
 
   // ---- epilogue: normalise and store --------------------------------------
   T *op = static_cast<T *>(p.out) + (int64_t)q_begin * p.o_row + (int64_t)h * p.o_head;
+  float *op32 = static_cast<float *>(p.out) + (int64_t)q_begin * p.o_row + (int64_t)h * p.o_head;
 #pragma unroll
   for (int qt = 0; qt < QT; qt++) {
     const int row = wave_row0 + qt * 32 + c;
@@ -409,7 +413,12 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
 #pragma unroll
       for (int a = 0; a < 4; a++) {
         const int dcol = dt * 32 + a * 8 + g * 4;
-        if (dcol < p.d) {
+        if (dcol < p.d && p.out_f32) {
+          f32x4_t r;
+#pragma unroll
+          for (int i = 0; i < 4; i++) r[i] = acc[qt][dt][a * 4 + i] * inv;
+          *reinterpret_cast<f32x4_t *>(op32 + (int64_t)row * p.o_row + dcol) = r;
+        } else if (dcol < p.d) {
           T r[4];
 #pragma unroll
           for (int i = 0; i < 4; i++) r[i] = from_float<T>(acc[qt][dt][a * 4 + i] * inv);
@@ -938,7 +947,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         if (i > 0) mx = max3(mx, s[0][i], s[1][i]);
     }
     mx = max_across_halves(mx) * p.scale_log2;
-    const bool grow = mx > m_run + kRescaleThreshold;
+    const bool grow = mx > m_run + p.rescale_thr;
     if (__builtin_expect(__any(grow), 0)) {
       const float m_new = grow ? mx : m_run;
       const float alpha = grow ? fast_exp2(m_run - m_new) : 1.0f;
@@ -1061,6 +1070,30 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   const int c_e = lane_e & 31, g_e = lane_e >> 5;
   const int wave_row0_e = wg_row0 + (wave_e < 4 ? wave_e : 11 - wave_e) * 32;
   T *ost = smem + wave_e * (32 * OSTR);
+  if (p.out_f32) {
+    // the checking form of the output: straight from the accumulators, 16 bytes per lane
+    float *op32 = static_cast<float *>(p.out) + (int64_t)q_begin * p.o_row + (int64_t)h * p.o_head;
+    const int row = wave_row0_e + c_e;
+    if (row < Lq) {
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+          const int dcol = dt * 32 + a * 8 + g_e * 4;
+          if (dcol < p.d) {
+            f32x4_t r;
+#pragma unroll
+            for (int i = 0; i < 4; i++) r[i] = acc[dt][a * 4 + i] * inv;
+            *reinterpret_cast<f32x4_t *>(op32 + (int64_t)row * p.o_row + dcol) = r;
+          }
+        }
+    }
+    if (p.lse != nullptr && g_e == 0 && row < Lq) {
+      const float lse = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : INFINITY;
+      p.lse[((int64_t)b * p.Hq + h) * p.lse_pitch + row] = lse;
+    }
+    return;
+  }
 #pragma unroll
   for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
@@ -1171,12 +1204,13 @@ __global__ void zero_kernel(T *ptr, int64_t rows, int64_t heads, int64_t d, int6
   }
 }
 
-void check_qkv(const hipattn_tensor *t, const char *name, int dtype, int d) {
+void check_qkv(const hipattn_tensor *t, const char *name, int dtype, int d, bool or_f32 = false) {
   check_tensor(t, name, 3);
-  HA_CHECK(t->dtype == dtype, "mha_varlen_fwd: %s dtype differs from q", name);
+  HA_CHECK(t->dtype == dtype || (or_f32 && t->dtype == HIPATTN_F32), "mha_varlen_fwd: %s dtype differs from q", name);
   HA_CHECK(t->sizes[2] == d, "mha_varlen_fwd: %s head size %lld differs from q's %d", name, (long long)t->sizes[2], d);
   HA_CHECK(d <= 1 || t->strides[2] == 1, "mha_varlen_fwd: %s must have a contiguous last dimension", name);
-  HA_CHECK(t->strides[0] % 8 == 0 && t->strides[1] % 8 == 0 && (reinterpret_cast<uintptr_t>(t->data) & 15) == 0,
+  const int per16 = 16 / dtype_size(t->dtype);
+  HA_CHECK(t->strides[0] % per16 == 0 && t->strides[1] % per16 == 0 && (reinterpret_cast<uintptr_t>(t->data) & 15) == 0,
            "mha_varlen_fwd: %s rows and heads must be 16-byte aligned", name);
   check_data(t, name);
 }
@@ -1195,7 +1229,7 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
   check_qkv(q, "q", q->dtype, d);
   check_qkv(k, "k", q->dtype, d);
   check_qkv(v, "v", q->dtype, d);
-  check_qkv(out, "out", q->dtype, d);
+  check_qkv(out, "out", q->dtype, d, true);
   const int Hkv = (int)k->sizes[1];
   HA_CHECK(v->sizes[0] == k->sizes[0] && v->sizes[1] == Hkv, "mha_varlen_fwd: k and v shapes differ");
   HA_CHECK(Hkv > 0 && Hq % Hkv == 0, "mha_varlen_fwd: %d query heads not divisible by %d kv heads", Hq, Hkv);
@@ -1233,7 +1267,9 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
   hipStream_t stream = resolve_stream(stream_arg);
   const int64_t total_q = q->sizes[0];
   if (zero_tensors && total_q > 0 && Hq > 0) {
-    if (q->dtype == HIPATTN_F16)
+    if (out->dtype == HIPATTN_F32)
+      zero_kernel<float><<<1024, 256, 0, stream>>>(static_cast<float *>(out->data), total_q, Hq, d, out->strides[0], out->strides[1]);
+    else if (q->dtype == HIPATTN_F16)
       zero_kernel<half_t><<<1024, 256, 0, stream>>>(static_cast<half_t *>(out->data), total_q, Hq, d, out->strides[0], out->strides[1]);
     else
       zero_kernel<bf16_t><<<1024, 256, 0, stream>>>(static_cast<bf16_t *>(out->data), total_q, Hq, d, out->strides[0], out->strides[1]);
@@ -1274,6 +1310,8 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
   p.causal = causal ? 1 : 0;
   p.win_left = win_left;
   p.win_right = win_right;
+  p.out_f32 = out->dtype == HIPATTN_F32 ? 1 : 0;
+  p.rescale_thr = (float)tuning().prefill_rescale_log2;
   if (q->dtype == HIPATTN_F16) dispatch_hd<half_t>(p, total_q, stream);
   else dispatch_hd<bf16_t>(p, total_q, stream);
 }
@@ -1312,7 +1350,7 @@ void mha_varlen_fwd_paged_impl(const hipattn_tensor *q, const hipattn_tensor *ke
   const int Hq = (int)q->sizes[1];
   HA_CHECK(d % 8 == 0 && d > 0 && d <= 128, "%s: head size must be a multiple of 8 in (0, 128], got %d", op, d);
   check_qkv(q, "q", q->dtype, d);
-  check_qkv(out, "out", q->dtype, d);
+  check_qkv(out, "out", q->dtype, d, true);
   HA_CHECK(out->sizes[0] == q->sizes[0] && out->sizes[1] == Hq, "%s: out shape differs from q", op);
   check_tensor(key_cache, "key_cache", 5);
   check_tensor(value_cache, "value_cache", 4);
@@ -1387,6 +1425,8 @@ void mha_varlen_fwd_paged_impl(const hipattn_tensor *q, const hipattn_tensor *ke
   p.causal = causal ? 1 : 0;
   p.win_left = -1;
   p.win_right = causal ? 0 : -1;
+  p.out_f32 = out->dtype == HIPATTN_F32 ? 1 : 0;
+  p.rescale_thr = (float)tuning().prefill_rescale_log2;
   p.block_tables = static_cast<const int32_t *>(block_tables->data);
   p.context_lens = static_cast<const int32_t *>(context_lens->data);
   p.table_stride = block_tables->strides[0];

@@ -70,8 +70,10 @@ const char *hipattn_version(void);
 /* Replaces mha_varlen_fwd_C (lib.rs:29-47; flash_api.cpp:447-655).
  * q [total_q, Hq, d], k/v [total_k, Hkv, d] (last dim contiguous, row and head
  * strides honoured), cu_seqlens_* int32 [b+1], seqused_k int32 [b] or NULL,
- * out [total_q, Hq, d] caller-allocated, softmax_lse f32 [b, Hq, max_seqlen_q]
- * or NULL.  fp16/bf16, d % 8 == 0, d <= 256, Hq % Hkv == 0.  Causal masking is
+ * out [total_q, Hq, d] caller-allocated, in q's dtype or f32 (the accumulators
+ * divided by the row sums and not rounded again: the form in which the
+ * kernel's arithmetic can be checked apart from the rounding of its output),
+ * softmax_lse f32 [b, Hq, max_seqlen_q] or NULL.  fp16/bf16 inputs, d % 8 == 0, d <= 256, Hq % Hkv == 0.  Causal masking is
  * bottom-right aligned: key j is visible to query i iff j <= i + (Lk - Lq)
  * (flash_attn/softmax.h:159-160).  window_size_left / window_size_right as in
  * the reference (flash_api.cpp:113-120,466; softmax.h:155-166): with bounds
@@ -99,7 +101,7 @@ char *hipattn_mha_varlen_fwd(const hipattn_tensor *q, const hipattn_tensor *k,
  * is in block block_tables[i][p / 16] at offset p % 16 (the new tokens' K/V
  * must already be in the cache); cu_seqlens_q int32 [b+1]; context_lens int32
  * [b] = keys per sequence; causal mask bottom-right aligned as in
- * hipattn_mha_varlen_fwd.  fp16/bf16, d % 8 == 0, d <= 128, block size 16. */
+ * hipattn_mha_varlen_fwd; out in q's dtype or f32 as there.  fp16/bf16, d % 8 == 0, d <= 128, block size 16. */
 char *hipattn_mha_varlen_fwd_paged(const hipattn_tensor *q, const hipattn_tensor *key_cache,
                                    const hipattn_tensor *value_cache, const hipattn_tensor *block_tables,
                                    const hipattn_tensor *cu_seqlens_q, const hipattn_tensor *context_lens,
@@ -400,7 +402,11 @@ char *hipattn_shutdown(void);
  * call, else 2..64), prefill_kernel (0 library's choice, 1 eight wavefronts,
  * 2 / 3 four wavefronts with 2 / 1 row tiles), paged_prefill_dma (-1 library's
  * choice, 0 staged tiles), cache_move_lds (-1 library's choice, 0 never the
- * LDS-transposing kernels).  Every setting computes the same results.  Not
+ * LDS-transposing kernels), prefill_rescale_log2 (0..16, default 8: the prefill
+ * kernels move a row's reference maximum only when the row outgrows it by
+ * more than 2^value; 0 follows the row maximum exactly, as the reference
+ * does).  Every setting computes the same results, prefill_rescale_log2 up to
+ * rounding.  Not
  * synchronised with running calls: set them between calls. */
 char *hipattn_tuning_set(const char *name, int value);
 char *hipattn_tuning_get(const char *name, int *value);

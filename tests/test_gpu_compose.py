@@ -124,10 +124,14 @@ def test_all_prefill_and_all_decode_steps(device):
     assert (y.float() - want).abs().max().item() <= TOL[torch.float16]
 
 
-def test_config4_full_size_sampled(device):
+@pytest.mark.parametrize("layout,paged_prefill", [("contiguous", False), ("fused_qkv", False), ("fused_qkv", True)])
+def test_config4_full_size_sampled(device, layout, paged_prefill):
     """The benchmark's mixed step at full size: 4 x 512-token chunks after 0/1k/2k/3k cached
-    tokens + 120 decode rows with contexts U[1k, 8k], 32 MHA heads, d 80, fp16.  The oracle runs
-    on the 4 chunks' last rows and a sample of decode rows (every row is independent)."""
+    tokens + 120 decode rows with contexts U[1k, 8k], 32 MHA heads, d 80, fp16 -- with contiguous
+    q, k, v and with q, k, v as views of one fused [T, 3, H, d] projection (token stride 3*H*d, what
+    Phi's layer passes, phi.rs:131-145), the latter also with the multi-token rows reading the cache
+    through block tables.  The oracle runs on the 4 chunks' last rows and a sample of decode rows
+    (every row is independent)."""
     rng = np.random.default_rng(4)
     g = torch.Generator().manual_seed(4)
     Hq = Hkv = 32
@@ -155,7 +159,13 @@ def test_config4_full_size_sampled(device):
     q = torch.randn((T, Hq, d), generator=g).to(dtype)
     k = torch.randn((T, Hkv, d), generator=g).to(dtype)
     v = torch.randn((T, Hkv, d), generator=g).to(dtype)
-    y = attn.varlen_attn(q.to(device), k.to(device), v.to(device), bi.to(device), kd, vd).reshape(T, Hq, d)
+    if layout == "fused_qkv":
+        qkv = torch.stack([q, k, v], dim=1).to(device)
+        qd, kin, vin = qkv[:, 0], qkv[:, 1], qkv[:, 2]
+        assert qd.stride(0) == 3 * Hq * d
+    else:
+        qd, kin, vin = q.to(device), k.to(device), v.to(device)
+    y = attn.varlen_attn(qd, kin, vin, bi.to(device), kd, vd, paged_prefill=paged_prefill).reshape(T, Hq, d)
     assert not torch.isnan(y.float()).any()
     kc, vc = kd.cpu(), vd.cpu()  # after the step: holds the new tokens too
     worst = 0.0

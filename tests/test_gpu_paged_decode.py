@@ -367,3 +367,35 @@ def test_context_lengths_above_the_stated_maximum_are_cut_there(device, dtype, b
     tol = FP32_TOL if dtype == torch.float32 else TOL[dtype]
     assert not torch.isnan(out).any()
     assert (out.cpu().float() - want).abs().max().item() <= tol
+
+
+def test_config5_decode_shape(device):
+    """The decode attention of the full-model configuration at its own shape: 128 sequences with contexts
+    U[1024, 16384] (seed 5), 32 q / 8 kv heads, d 128, bf16 -- 1.1 M context tokens, 4.6 GB of K/V in a
+    70k-block pool.  The cache is filled on the GPU (seeded); 18 sequences, the shortest and the longest
+    among them, are checked against the oracle on their own blocks brought to the CPU, all 128 by the range
+    property (an attention output is a convex combination of its context's V rows)."""
+    rng = np.random.default_rng(5)
+    S = 128
+    ctx = rng.integers(1024, 16384 + 1, size=S)
+    pool = int(((ctx + 15) // 16).sum()) + 64
+    c = W.decode_inputs(5, S, 1024, 16384, 32, 8, 128, torch.bfloat16, pool, device=device)
+    assert np.array_equal(c.context_lens.cpu().numpy(), ctx.astype(np.int32))   # the same draw as the benchmark's
+    out = torch.full_like(c.q, float("nan"))
+    K.paged_attention_v1(out, c.q, c.key_cache, c.value_cache, 8, c.scale, c.block_tables, c.context_lens, 16,
+                         c.max_ctx)
+    assert not torch.isnan(out).any()
+    assert out.float().abs().max().item() <= c.value_cache.float().abs().max().item()
+    rows = sorted({int(np.argmin(ctx)), int(np.argmax(ctx)), *range(0, S, 8)})
+    assert len(rows) >= 16
+    if "config5" not in _ORACLE_CACHE:
+        want = []
+        for s in rows:
+            n = (int(ctx[s]) + 15) // 16
+            blocks = c.block_tables[s, :n].long()
+            kc, vc = c.key_cache[blocks].cpu(), c.value_cache[blocks].cpu()   # this sequence's blocks, renumbered 0..n-1
+            want.append(ref.paged_attention(c.q[s:s + 1].cpu().float(), kc.float(), vc.float(), 8, c.scale,
+                                            torch.arange(n, dtype=torch.int32)[None], c.context_lens[s:s + 1].cpu(), 16)[0])
+        _ORACLE_CACHE["config5"] = torch.stack(want)
+    err = (out[rows].cpu().float() - _ORACLE_CACHE["config5"]).abs().max().item()
+    assert err <= TOL[torch.bfloat16], err

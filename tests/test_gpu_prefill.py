@@ -139,22 +139,61 @@ def test_strided_qkv_from_a_fused_projection(device):
     assert (got.cpu().double() - fp64(p)).abs().max().item() <= TOL[dtype]
 
 
+def bf16_half_ulp(x: torch.Tensor) -> torch.Tensor:
+    """Half the spacing of bf16 numbers at |x| (8 significand bits): what storing x as bf16 can cost."""
+    return torch.maximum(x.abs(), torch.tensor(2.0 ** -126, dtype=x.dtype)).log2().floor().exp2() * 2.0 ** -8
+
+
 @pytest.mark.parametrize("sigma", [1.0, 2.0])
 def test_config3_shape_reduced_against_fp64(device, sigma):
-    """Llama-3-8B attention shape (32 q / 8 kv heads, d 128, bf16), 2 x 1024 tokens, N(0,1) and N(0,4)."""
+    """Llama-3-8B attention shape (32 q / 8 kv heads, d 128, bf16), 2 x 1024 tokens, N(0,1) and N(0,4),
+    every element against the fp64 statement.  The 2e-2 gate is applied, as it stands, to the kernel's
+    fp32 output (its arithmetic: bf16 operands, fp32 accumulation, division by the row sum).  The bf16
+    output is that value rounded once more; with N(0,4) inputs |o| passes 8, where a bf16 cannot be
+    closer than 0.031 to an arbitrary number, so for it the test reports the error next to max |ref| and
+    the number of elements whose own rounding step exceeds the gate, and requires the error to stay
+    within gate + that step."""
+    gate = TOL[torch.bfloat16]
     p = W.config3(sigma, batch=2, L=1024)
-    got = run(p, device).cpu()
     want = fp64(p)
+    got32 = run(p, device, out_dtype=torch.float32).cpu()
+    assert got32.dtype == torch.float32
+    err32 = (got32.double() - want).abs().max().item()
+    assert err32 <= gate, (sigma, err32)
+    got = run(p, device).cpu()
+    # the bf16 output is the fp32 output rounded to nearest-even, nothing else
+    assert torch.equal(got, got32.to(torch.bfloat16))
     err = (got.double() - want).abs()
+    step = bf16_half_ulp(want)
+    beyond = int((step > gate).sum())
+    print(f"sigma {sigma}: fp32-output max-abs err {err32:.3e}; bf16-output max-abs err {err.max().item():.3e}, "
+          f"max |ref| {want.abs().max().item():.2f}, elements whose bf16 half-ulp exceeds the gate: {beyond}")
     if sigma == 1.0:
-        assert err.max().item() <= TOL[torch.bfloat16]
+        assert beyond == 0 and err.max().item() <= gate
     else:
-        # With N(0,4) inputs |o| reaches 8 and beyond, where storing a bf16 costs up to half an
-        # ulp = 0.0156 (4 <= |o| < 8) or 0.031 (>= 8): the absolute gate is applied to what the
-        # kernel can control, the error beyond the output's own rounding step.
-        half_ulp = torch.maximum(want.abs(), torch.tensor(1.0)).log2().floor().exp2() * 2.0 ** -8
-        assert (err - half_ulp).max().item() <= TOL[torch.bfloat16]
-        assert (err <= TOL[torch.bfloat16]).double().mean().item() > 0.9999
+        assert (err - step).max().item() <= gate
+
+
+def test_config3_full_size_sampled_rows_wide_inputs(device):
+    """8 x 4096 with N(0,4) inputs (the softmax-range stress of config 3): sampled rows of the fp32 output
+    against fp64 with the plain gate; the bf16 output is the same numbers rounded."""
+    p = W.config3(2.0, device=device)
+    out32 = K.flash_attn_varlen(p.q, p.k, p.v, p.cu_q, p.cu_k, p.max_q, p.max_k, p.scale, True, out_dtype=torch.float32)
+    out = K.flash_attn_varlen(p.q, p.k, p.v, p.cu_q, p.cu_k, p.max_q, p.max_k, p.scale, True)
+    assert torch.equal(out, out32.to(torch.bfloat16))
+    rng = np.random.default_rng(1)
+    rows = [(0, 0, 0), (7, 31, 4095), (2, 9, 255), (2, 9, 256), (5, 20, 2047), (5, 20, 2048)]
+    rows += [(int(rng.integers(8)), int(rng.integers(32)), int(rng.integers(4096))) for _ in range(90)]
+    worst, worst_ref = 0.0, 0.0
+    for b, h, i in rows:
+        qrow = p.q[b * 4096 + i, h].double()
+        keys = p.k[b * 4096:b * 4096 + i + 1, h // 4].double()
+        vals = p.v[b * 4096:b * 4096 + i + 1, h // 4].double()
+        ref_row = torch.softmax(keys @ qrow * p.scale, 0) @ vals
+        worst = max(worst, (out32[b * 4096 + i, h].double() - ref_row).abs().max().item())
+        worst_ref = max(worst_ref, ref_row.abs().max().item())
+    print(f"N(0,4) 8 x 4096, {len(rows)} rows: fp32-output max-abs err {worst:.3e}, max |ref| {worst_ref:.2f}")
+    assert worst <= TOL[torch.bfloat16], worst
 
 
 def test_config3_full_size_sampled_rows(device):

@@ -171,3 +171,18 @@ def test_blocks_beyond_4_gib_of_cache(device):
     one = W.offsets([1] * len(seqs)).to(device)
     want_d = K.flash_attn_varlen(qd, k, v, one, cu_k, 1, max(lens_k), scale, True)
     assert (out.float() - want_d.float()).abs().max().item() <= TOL[dtype]
+
+
+@pytest.mark.parametrize("heads", [(32, 8, 128), (32, 32, 80)])
+def test_fp32_output_is_the_unrounded_result(device, heads):
+    """out in f32: the accumulators divided by the row sums; rounding it gives the bf16 output bit for bit,
+    and it is closer to the oracle than the rounded one."""
+    Hq, Hkv, d = heads
+    c = paged_case(35, SEQS, Hq, Hkv, d, torch.bfloat16, 420)
+    args = (c["q"].to(device), c["kc"].to(device), c["vc"].to(device), c["tables"].to(device), c["cu_q"].to(device),
+            c["ctx"].to(device), max(c["lens_q"]), max(c["lens_k"]), c["scale"], True)
+    got32 = K.flash_attn_varlen_paged(*args, out_dtype=torch.float32)
+    got = K.flash_attn_varlen_paged(*args)
+    assert got32.dtype == torch.float32 and torch.equal(got, got32.to(torch.bfloat16))
+    want = oracle(c, Hq, Hkv, d)
+    assert (got32.cpu() - want).abs().max().item() <= (got.cpu().float() - want).abs().max().item() <= TOL[torch.bfloat16]
