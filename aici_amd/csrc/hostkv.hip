@@ -260,6 +260,20 @@ extern "C" char *hipattn_block_allocator_swap_in(hipattn_block_allocator *a, int
              (long long)seq_id);
     HA_CHECK(*n_pairs >= 0 && *n_pairs <= pair_capacity && (pair_capacity == 0 || mapping != nullptr),
              "swap_in: bad mapping buffer");
+    // Count what the call will take before it takes anything, so that a failure leaves the allocator and
+    // the mapping as they were: every entry not yet mapped -- by the group so far or earlier in this list --
+    // needs one free block and one pair.
+    int64_t fresh = 0;
+    for (int64_t i = 0; i < n; i++) {
+      bool known = false;
+      for (int64_t k = 0; k < *n_pairs && !known; k++) known = mapping[2 * k] == block_idxs[i];
+      for (int64_t j = 0; j < i && !known; j++) known = block_idxs[j] == block_idxs[i];
+      if (!known) fresh++;
+    }
+    HA_CHECK(*n_pairs + fresh <= pair_capacity, "swap_in: mapping buffer too small (%lld pairs, %lld needed)",
+             (long long)pair_capacity, (long long)(*n_pairs + fresh));
+    HA_CHECK((int64_t)a->free_list.size() >= fresh, "Out of memory! swap_in needs %lld free blocks, %lld are available.",
+             (long long)fresh, (long long)a->free_list.size());
     std::vector<int64_t> v;
     v.reserve((size_t)n);
     for (int64_t i = 0; i < n; i++) {

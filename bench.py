@@ -5,10 +5,14 @@
 Headline (`value`): paged decode attention over the benchmark's decode configuration
 (64 sequences, contexts U[512,4096], 32 q / 8 kv heads, d 128, bf16, block size 16, tables from
 a shuffled 20k-block pool) as algorithmic HBM GB/s, with inputs resident in HBM.  One step = one
-`paged_attention_v1` call over the batch.  The same line also carries the prefill leg
-(`prefill`: 8 x 4096 GQA causal varlen prefill, TFLOP/s against the bf16 MFMA peak) and the CPU
-baseline (`cpu_baseline`: the oracle, i.e. rLLM's CPU reference route restated in torch-CPU,
-timed on a bounded sample of the same workload on this box's host cores).
+`paged_attention_v1` call over the batch (both of its kernels).  The block of `--steps` steps is
+repeated until at least 100 ms have been timed; `value` is the median block, the spread is reported.
+The same line carries the other configurations: `prefill` (8 x 4096 GQA causal varlen prefill,
+TFLOP/s against the bf16 MFMA peak, with its own CPU baseline), `mixed_step` (the Phi-2-shaped
+continuous-batching step), `llama_step` (the full Llama-3-8B-shaped decode step with the AICI mask),
+`memory_system` (what plain read / copy / fill kernels reach on this device) and `cpu_baseline`
+(the oracle, i.e. rLLM's CPU reference route restated in torch-CPU, timed on a bounded sample of
+the decode workload on this box's host cores).
 """
 from __future__ import annotations
 
@@ -23,10 +27,82 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
-# HBM bytes per decode launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB
-# copy (profiles/decode_c2_hbm_traffic.md); bench.py cannot read counters itself.
-DECODE_TRAFFIC_BYTES = 643.2e6
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
+# Figures bench.py cannot measure itself (hardware counters, single kernels of a multi-kernel step):
+# taken from the rocprofv3 summaries under profiles/, which name the commands that made them.
+PROFILED = {
+    "decode_traffic_bytes": 643.2e6,      # FETCH_SIZE + WRITE_SIZE per decode step, scaled by a 1 GiB copy
+    "decode_traffic_source": "profiles/decode_c2_hbm_traffic.md",
+    "decode_main_kernel_us": 118.9,       # paged_decode_flat_kernel, average duration in the kernel trace
+    "decode_reduce_kernel_us": 5.1,       # paged_decode_flat_reduce_kernel
+    "decode_kernels_source": "profiles/decode_c2_prefill_c3_kernel_trace.md",
+    "prefill_traffic_bytes": None,
+    "prefill_traffic_source": None,
+}
+MIN_TIMED_MS = 100.0
+
+
+def timed_blocks(fn, steps: int, min_total_ms: float = MIN_TIMED_MS, max_blocks: int = 400) -> list:
+    """Wall time per step (ms) of blocks of exactly `steps` calls, each block bracketed by a device
+    synchronisation on both sides; blocks are repeated until `min_total_ms` of timed work has run."""
+    import torch
+
+    per_step, total = [], 0.0
+    while (total < min_total_ms or len(per_step) < 3) and len(per_step) < max_blocks:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) * 1e3
+        per_step.append(dt / steps)
+        total += dt
+    return per_step
+
+
+def spread(xs: list) -> dict:
+    import statistics
+
+    return {"blocks": len(xs), "median": round(statistics.median(xs), 5), "min": round(min(xs), 5),
+            "max": round(max(xs), 5)}
+
+
+def host_cores() -> dict:
+    """Cores this process may run on and cores the box reports (a container's share can be smaller)."""
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    # a one-GPU box of this pool shares its host: 16 cores go with one GPU, whatever the counts above say
+    return {"usable": usable, "reported": os.cpu_count() or 1, "share_for_one_gpu": 16, "threads_used": min(usable, 16)}
+
+
+def cpu_baseline_prefill(p_cpu, seq: int, threads: int) -> dict:
+    """The oracle's varlen attention (repeat_kv -> per-sequence fp32 SDPA with an additive causal bias, the
+    route of rLLM's CPU build) on one of the prefill configuration's sequences."""
+    import torch
+
+    from oracle import refkernels as ref
+
+    torch.set_num_threads(threads)
+    L = p_cpu.lens_q[seq]
+    a, b = int(p_cpu.cu_q[seq]), int(p_cpu.cu_q[seq + 1])
+    q, k, v = p_cpu.q[a:b].float(), p_cpu.k[a:b].float(), p_cpu.v[a:b].float()
+    n_rep = q.shape[1] // k.shape[1]
+    cu = torch.tensor([0, L], dtype=torch.int32)
+    reps, dt = 0, 0.0
+    t0 = time.perf_counter()
+    while dt < 10.0:  # a bounded sample: about 10 s of CPU work
+        ref.varlen_attn(q, ref.repeat_kv(k, n_rep), ref.repeat_kv(v, n_rep), cu, cu, L, L, p_cpu.scale, True)
+        reps += 1
+        dt = time.perf_counter() - t0
+    dt /= reps
+    flops = 4.0 * q.shape[2] * q.shape[1] * (L * (L + 1) // 2)
+    return {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"sequence {seq} of {len(p_cpu.lens_q)} ({L} tokens; every sequence costs the same), {reps} "
+                      f"passes of {dt:.2f} s; flops counted as for the GPU (unmasked pairs only, although the CPU "
+                      "route computes the full L x L products)"}
+
 
 
 def event_times_ms(fn, steps: int, stream) -> list:
@@ -311,13 +387,16 @@ def main() -> None:
     ap.add_argument("--streaming", action="store_true",
                     help="also time the HBM-bound helper kernels (cache scatter/gather, rotary, norms, "
                          "activation, bias + arg-max) against the HBM roofline")
-    ap.add_argument("--mixed-step", action="store_true",
-                    help="also time one layer's attention for a mixed prefill-chunk + decode step (Phi-2 shape)")
-    ap.add_argument("--llama-step", action="store_true",
-                    help="also time a full Llama-3-8B-shaped decode step with the AICI mask + greedy stage "
-                         "(allocates about 170 GB of HBM)")
+    ap.add_argument("--no-mixed-step", action="store_true",
+                    help="skip one layer's attention for the mixed prefill-chunk + decode step (Phi-2 shape)")
+    ap.add_argument("--no-llama-step", action="store_true",
+                    help="skip the full Llama-3-8B-shaped decode step with the AICI mask + greedy stage "
+                         "(it allocates about 170 GB of HBM)")
+    ap.add_argument("--mixed-step", action="store_true", help="(default; kept for old command lines)")
+    ap.add_argument("--llama-step", action="store_true", help="(default; kept for old command lines)")
     ap.add_argument("--llama-layers", type=int, default=32)
-    ap.add_argument("--llama-share-cache", action="store_true", help="all layers read one layer's KV cache")
+    ap.add_argument("--llama-share-cache", action="store_true",
+                    help="all layers read one layer's KV cache (taken by itself when the device is short of memory)")
     ap.add_argument("--no-memory-system", action="store_true",
                     help="skip the plain read / copy / fill kernels and the shuffled 4 KiB-chunk read (the "
                          "attainable rates reported beside the 8 TB/s peak)")
@@ -339,6 +418,7 @@ def main() -> None:
         sys.exit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     stream = torch.cuda.current_stream(dev)
+    K.init()
 
     # ---- decode leg (headline) ------------------------------------------------------------
     c_cpu = W.config2()
@@ -357,22 +437,19 @@ def main() -> None:
         K.paged_attention_v1(out, c.q, kc, vc, c.num_kv_heads, c.scale, c.block_tables, c.context_lens, 16,
                              c.max_ctx)
 
-    for _ in range(args.warmup):
+    for _ in range(max(args.warmup, 1)):
         decode_step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        decode_step()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    step_ms = event_times_ms(decode_step, args.steps, stream)
+    wall = timed_blocks(decode_step, args.steps)
+    import statistics
+
+    wall_ms = statistics.median(wall)
+    # HIP events on the launch stream around every step (both kernels of the call)
+    step_ms = event_times_ms(decode_step, max(args.steps, 100), stream)
     avg_step_ms = sum(step_ms) / len(step_ms)
-    # The dominant kernel on its own: the same launches with the (small) merge kernel left out, which is
-    # what `roofline.achieved` is defined on; `value` above is the whole step.
-    avg_launch_ms = avg_step_ms
     nbytes = c_cpu.algorithmic_bytes()
     value = nbytes / (wall_ms * 1e-3) / 1e9
-    achieved = nbytes / (avg_launch_ms * 1e-3) / 1e9
+    achieved = nbytes / (avg_step_ms * 1e-3) / 1e9
+    main_us = PROFILED["decode_main_kernel_us"]
 
     line = {
         "metric": "prefill attn TFLOP/s + paged-decode attn HBM GB/s (1 GPU, % roofline)",
@@ -382,6 +459,7 @@ def main() -> None:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(wall_ms, 5),
+        "ms_per_step_spread": spread(wall),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -392,11 +470,18 @@ def main() -> None:
                    "algorithmic_bytes_per_step": nbytes,
                    "context_tokens": int(c_cpu.context_lens.sum()), "kv_pool_copies": len(pools)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": DECODE_TRAFFIC_BYTES,
-                     "kernel": "paged_decode_flat_kernel alone (merge kernel left out for this measurement), "
-                               "HIP events on the launch stream",
-                     "avg_launch_us": round(avg_launch_ms * 1e3, 2),
-                     "avg_step_us_with_merge_kernel": round(avg_step_ms * 1e3, 2)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": PROFILED["decode_traffic_bytes"],
+                     "traffic_source": PROFILED["decode_traffic_source"],
+                     "kernel": "the whole decode step: paged_decode_flat_kernel + paged_decode_flat_reduce_kernel, "
+                               "HIP events on the launch stream around each call",
+                     "avg_step_us": round(avg_step_ms * 1e3, 2),
+                     "dominant_kernel_alone": {
+                         "kernel": "paged_decode_flat_kernel", "avg_launch_us": main_us,
+                         "achieved": round(nbytes / main_us / 1e3, 1),
+                         "frac": round(nbytes / main_us / 1e3 / HBM_PEAK_GBS, 4),
+                         "source": PROFILED["decode_kernels_source"] + " (rocprofv3 kernel trace of this command; "
+                                   "not measured in this run)"}},
+        "host_cores": host_cores(),
     }
 
     if args.copy_calibration:
@@ -410,7 +495,8 @@ def main() -> None:
 
     # ---- prefill leg ------------------------------------------------------------------------
     if not args.no_prefill:
-        p = W.config3(1.0, device=dev)
+        p_cpu = W.config3(1.0)
+        p = p_cpu.to(dev)
 
         def prefill_step():
             K.flash_attn_varlen(p.q, p.k, p.v, p.cu_q, p.cu_k, p.max_q, p.max_k, p.scale, True)
@@ -419,17 +505,20 @@ def main() -> None:
         psteps = max(3, min(args.steps, 50))
         for _ in range(max(25, args.warmup)):
             prefill_step()
-        torch.cuda.synchronize()
+        pwall = timed_blocks(prefill_step, psteps)
         pl = event_times_ms(prefill_step, psteps, stream)
         pms = sum(pl) / len(pl)
         tflops = p.flops() / (pms * 1e-3) / 1e12
         line["prefill"] = {
-            "value": round(tflops, 1), "unit": "TFLOP/s", "ms_per_step": round(pms, 4), "steps": psteps,
+            "value": round(p.flops() / (statistics.median(pwall) * 1e-3) / 1e12, 1), "unit": "TFLOP/s",
+            "ms_per_step": round(statistics.median(pwall), 4), "ms_per_step_spread": spread(pwall), "steps": psteps,
             "config": {"workload": "varlen causal prefill: 8 x 4096 tokens, 32 q / 8 kv heads, d 128, bf16, N(0,1)",
                        "algorithmic_flops_per_step": p.flops()},
             "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
-                         "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                         "kernel": "prefill_varlen_w8_kernel, HIP events on the launch stream"},
+                         "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                         "traffic": PROFILED["prefill_traffic_bytes"], "traffic_source": PROFILED["prefill_traffic_source"],
+                         "kernel": "prefill_varlen_w8_kernel, HIP events on the launch stream",
+                         "avg_launch_us": round(pms * 1e3, 1)},
         }
         # The same rows with K/V read from the paged cache they were scattered into (what an engine step
         # has at hand: rLLM writes the cache first, llm/mod.rs:147-164, and gathers back from it).
@@ -452,7 +541,7 @@ def main() -> None:
         for _ in range(10):
             paged_step()
         torch.cuda.synchronize()
-        ql = event_times_ms(paged_step, psteps, stream)
+        ql = event_times_ms(paged_step, max(psteps, 90), stream)
         qms = sum(ql) / len(ql)
         line["prefill"]["from_paged_cache"] = {
             "value": round(p.flops() / (qms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": round(qms, 4),
@@ -465,22 +554,33 @@ def main() -> None:
         line["streaming"] = streaming_leg(dev, stream, max(20, min(args.steps, 100)))
 
     if not args.no_memory_system:
-        line["memory_system"] = memory_system_leg(dev, stream, 20)
+        line["memory_system"] = memory_system_leg(dev, stream, 100)
 
-    if args.mixed_step:
-        line["mixed_step"] = mixed_step_leg(dev, stream, max(20, min(args.steps, 100)))
+    if not args.no_mixed_step:
+        line["mixed_step"] = mixed_step_leg(dev, stream, max(100, args.steps))
 
-    # ---- optional: the full engine step the decode kernel sits in ---------------------------------
-    if args.llama_step:
+    # ---- the full engine step the decode kernel sits in -------------------------------------------
+    if not args.no_llama_step:
         del pools, c
         torch.cuda.empty_cache()
-        line["llama_step"] = llama_step_leg(dev, stream, max(3, min(args.steps, 10)), args.llama_layers,
-                                            args.llama_share_cache)
+        free_b, _total = torch.cuda.mem_get_info(dev)
+        need = 175e9 * args.llama_layers / 32
+        share = args.llama_share_cache or free_b < need
+        try:
+            line["llama_step"] = llama_step_leg(dev, stream, max(4, min(args.steps, 10)), args.llama_layers, share)
+            if share and not args.llama_share_cache:
+                line["llama_step"]["note"] = (f"one KV cache shared by all layers: {free_b / 1e9:.0f} GB free on the "
+                                              f"device, {need / 1e9:.0f} GB needed for a cache per layer")
+        except torch.OutOfMemoryError as e:
+            line["llama_step"] = {"skipped": f"out of device memory: {str(e)[:160]}"}
+        torch.cuda.empty_cache()
 
-    # ---- CPU baseline: the reference's CPU route on this box's host cores ------------------------
+    # ---- CPU baselines: the reference's CPU route on this box's host cores ------------------------
     if not args.no_cpu_baseline:
-        threads = min(os.cpu_count() or 1, 16)
+        threads = host_cores()["threads_used"]
         line["cpu_baseline"] = cpu_baseline_decode(c_cpu, list(range(0, 64, 2)), threads)
+        if "prefill" in line:
+            line["prefill"]["cpu_baseline"] = cpu_baseline_prefill(p_cpu, 0, threads)
 
     print(json.dumps(line), flush=True)
 
