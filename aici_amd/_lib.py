@@ -137,6 +137,15 @@ _ERR_FUNCS = {
                                   c_int64],
     "hipattn_batch_builder_add_seq": [c_void_p, c_void_p, c_int64, POINTER(c_int32), c_int64, c_int64],
     "hipattn_batch_builder_finish": [c_void_p, POINTER(BatchInfo)],
+    "hipattn_decode_batch_new": [c_int64, c_int64, POINTER(c_void_p)],
+    "hipattn_decode_batch_add": [c_void_p, c_void_p, c_int64, c_int32, c_int64],
+    "hipattn_decode_batch_advance": [c_void_p, c_void_p, c_int64, c_int32],
+    "hipattn_decode_batch_advance_all": [c_void_p, c_void_p, POINTER(c_int32), c_int64],
+    "hipattn_decode_batch_remove": [c_void_p, c_int64],
+    "hipattn_decode_batch_info": [c_void_p, POINTER(BatchInfo)],
+    "hipattn_block_allocator_step_generation": [c_void_p, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), c_int64,
+                                                POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
+                                                POINTER(c_int64), c_int64, POINTER(c_int64)],
     "hipattn_varlen_attn": [TP, TP, TP, TP, TP, TP, TP, TP, TP, c_int64, c_int, c_int, TP, TP, c_int, c_int, c_float,
                             TP, TP, TP, c_void_p],
     "hipattn_varlen_attn_paged": [TP, TP, TP, TP, TP, TP, TP, TP, TP, c_int64, c_int, c_int, TP, TP, c_int, c_int,
@@ -153,6 +162,8 @@ _PLAIN_FUNCS = {
     "hipattn_block_allocator_can_append_slot": (ctypes.c_int, [c_void_p, c_int64]),
     "hipattn_block_allocator_num_allocated": (c_int64, [c_void_p, c_int64]),
     "hipattn_batch_builder_free": (None, [c_void_p]),
+    "hipattn_decode_batch_free": (None, [c_void_p]),
+    "hipattn_decode_batch_size": (c_int64, [c_void_p]),
     "hipattn_cache_x": (c_int64, [c_int32]),
     "hipattn_cache_block_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_int32]),
 }

@@ -62,6 +62,23 @@ class BlockAllocator:
              cap, ctypes.byref(n))
         return [(int(buf[2 * i]), int(buf[2 * i + 1])) for i in range(n.value)]
 
+    def step_generation(self, seq_ids: Sequence[int], seq_lens: Sequence[int], num_kv_computed: Sequence[int]):
+        """scheduler.rs:304-337 + 357-380 for groups of one sequence (ids in arrival order): returns
+        (scheduled ids, preempted ids, copy-on-write pairs).  A preempted sequence holds no blocks any more
+        and has to be admitted and recomputed."""
+        n = len(seq_ids)
+        ids = (ctypes.c_int64 * max(1, n))(*[int(x) for x in seq_ids])
+        lens = (ctypes.c_int64 * max(1, n))(*[int(x) for x in seq_lens])
+        comp = (ctypes.c_int64 * max(1, n))(*[int(x) for x in num_kv_computed])
+        sched, pre = (ctypes.c_int64 * max(1, n))(), (ctypes.c_int64 * max(1, n))()
+        cap = sum((int(l) + self.block_size - 1) // self.block_size + 1 for l in seq_lens) + 1
+        pairs = (ctypes.c_int64 * (2 * cap))()
+        ns, np_, npairs = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+        call("hipattn_block_allocator_step_generation", self._h, ids, lens, comp, n, sched, ctypes.byref(ns), pre,
+             ctypes.byref(np_), pairs, cap, ctypes.byref(npairs))
+        return ([int(sched[i]) for i in range(ns.value)], [int(pre[i]) for i in range(np_.value)],
+                [(int(pairs[2 * i]), int(pairs[2 * i + 1])) for i in range(npairs.value)])
+
     def copy(self, src: int, dst: int, length: int) -> None:
         call("hipattn_block_allocator_copy", self._h, int(src), int(dst), int(length))
 
@@ -250,30 +267,74 @@ class BatchInfoBuilder:
     def finish(self) -> BatchInfo:
         bi = _lib.BatchInfo()
         call("hipattn_batch_builder_finish", self._h, ctypes.byref(bi))
-        nm = int(bi.num_multi)
-        tables = _np(bi.paged_block_tables, int(bi.num_paged * bi.paged_max_blocks), np.int32)
-        return BatchInfo(
-            tokens=torch.from_numpy(_np(bi.tokens, int(bi.num_tokens), np.int32)),
-            positions=torch.from_numpy(_np(bi.positions, int(bi.num_tokens), np.int64)),
-            seqlens_q=torch.from_numpy(_np(bi.seqlens_q, nm + 1, np.int32)),
-            seqlens_k=torch.from_numpy(_np(bi.seqlens_k, nm + 1, np.int32)),
-            gather_mapping=torch.from_numpy(_np(bi.gather_mapping, int(bi.num_gather), np.int32)),
-            slot_mapping=torch.from_numpy(_np(bi.slot_mapping, int(bi.num_tokens), np.int32)),
-            logit_idxs=torch.from_numpy(_np(bi.logit_idxs, int(bi.num_seqs), np.int32)),
-            max_seqlen_q=int(bi.max_seqlen_q),
-            max_seqlen_k=int(bi.max_seqlen_k),
-            seq_ids=[int(x) for x in _np(bi.seq_ids, int(bi.num_seqs), np.int64)],
-            paged_block_tables=torch.from_numpy(tables).reshape(int(bi.num_paged), int(bi.paged_max_blocks)),
-            paged_context_lens=torch.from_numpy(_np(bi.paged_context_lens, int(bi.num_paged), np.int32)),
-            paged_block_size=int(bi.paged_block_size),
-            paged_max_context_len=int(bi.paged_max_context_len),
-            seqlen_multi=nm,
-            q_multi=int(bi.q_multi),
-            multi_block_tables=(torch.from_numpy(_np(bi.multi_block_tables, nm * int(bi.multi_max_blocks), np.int32))
-                                .reshape(nm, int(bi.multi_max_blocks)) if bi.multi_tables_valid else None),
-            multi_context_lens=(torch.from_numpy(_np(bi.multi_context_lens, nm, np.int32))
-                                if bi.multi_tables_valid else None),
-        )
+        return _batch_info(bi)
+
+
+class DecodeBatch:
+    """The single-token rows of a running batch kept across steps (`hipattn_decode_batch`): `info()` equals
+    what `BatchInfoBuilder.finish()` gives for the same sequences in the same order, without the per-step
+    rebuild from every sequence's full slot list (batch_info.rs:196-315)."""
+
+    def __init__(self, block_size: int, max_model_len: int):
+        h = ctypes.c_void_p()
+        call("hipattn_decode_batch_new", int(block_size), int(max_model_len), ctypes.byref(h))
+        self._h = h
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h and _lib is not None:
+            _lib.load().hipattn_decode_batch_free(h)
+
+    def __len__(self) -> int:
+        return int(_lib.load().hipattn_decode_batch_size(self._h))
+
+    def add(self, alloc: BlockAllocator, seq_id: int, last_token: int, seq_len: int) -> None:
+        call("hipattn_decode_batch_add", self._h, alloc._h, int(seq_id), int(last_token), int(seq_len))
+
+    def advance(self, alloc: BlockAllocator, seq_id: int, new_token: int) -> None:
+        call("hipattn_decode_batch_advance", self._h, alloc._h, int(seq_id), int(new_token))
+
+    def advance_all(self, alloc: BlockAllocator, new_tokens: Sequence[int]) -> None:
+        """One generation step for every row: new_tokens[i] is row i's new token."""
+        t = np.ascontiguousarray(new_tokens, dtype=np.int32)
+        call("hipattn_decode_batch_advance_all", self._h, alloc._h, t.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)),
+             len(t))
+
+    def remove(self, seq_id: int) -> None:
+        call("hipattn_decode_batch_remove", self._h, int(seq_id))
+
+    def info(self) -> BatchInfo:
+        bi = _lib.BatchInfo()
+        call("hipattn_decode_batch_info", self._h, ctypes.byref(bi))
+        return _batch_info(bi)
+
+
+def _batch_info(bi) -> BatchInfo:
+    """Copies a `hipattn_batch_info` (arrays owned by the C++ side) into host tensors."""
+    nm = int(bi.num_multi)
+    tables = _np(bi.paged_block_tables, int(bi.num_paged * bi.paged_max_blocks), np.int32)
+    return BatchInfo(
+        tokens=torch.from_numpy(_np(bi.tokens, int(bi.num_tokens), np.int32)),
+        positions=torch.from_numpy(_np(bi.positions, int(bi.num_tokens), np.int64)),
+        seqlens_q=torch.from_numpy(_np(bi.seqlens_q, nm + 1, np.int32)),
+        seqlens_k=torch.from_numpy(_np(bi.seqlens_k, nm + 1, np.int32)),
+        gather_mapping=torch.from_numpy(_np(bi.gather_mapping, int(bi.num_gather), np.int32)),
+        slot_mapping=torch.from_numpy(_np(bi.slot_mapping, int(bi.num_tokens), np.int32)),
+        logit_idxs=torch.from_numpy(_np(bi.logit_idxs, int(bi.num_seqs), np.int32)),
+        max_seqlen_q=int(bi.max_seqlen_q),
+        max_seqlen_k=int(bi.max_seqlen_k),
+        seq_ids=[int(x) for x in _np(bi.seq_ids, int(bi.num_seqs), np.int64)],
+        paged_block_tables=torch.from_numpy(tables).reshape(int(bi.num_paged), int(bi.paged_max_blocks)),
+        paged_context_lens=torch.from_numpy(_np(bi.paged_context_lens, int(bi.num_paged), np.int32)),
+        paged_block_size=int(bi.paged_block_size),
+        paged_max_context_len=int(bi.paged_max_context_len),
+        seqlen_multi=nm,
+        q_multi=int(bi.q_multi),
+        multi_block_tables=(torch.from_numpy(_np(bi.multi_block_tables, nm * int(bi.multi_max_blocks), np.int32))
+                            .reshape(nm, int(bi.multi_max_blocks)) if bi.multi_tables_valid else None),
+        multi_context_lens=(torch.from_numpy(_np(bi.multi_context_lens, nm, np.int32))
+                            if bi.multi_tables_valid else None),
+    )
 
 
 _DT = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}

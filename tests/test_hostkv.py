@@ -284,3 +284,144 @@ def test_block_space_manager_admission_and_swaps():
     m.delete(3)
     m.trim(1, 16)
     assert m.get_num_free_gpu_blocks() == 299
+
+
+def test_swap_in_that_cannot_finish_changes_nothing():
+    a = paged.BlockAllocator(16, 4)
+    a.alloc_seq(1, 32)                      # two blocks taken, two free
+    mapping = {7: 0}
+    with pytest.raises(HipAttnError, match="needs 3 free blocks, 2 are available"):
+        a.swap_in(2, [7, 8, 9, 10, 8], mapping)   # 7 is mapped, 8 / 9 / 10 need fresh blocks
+    assert a.get_num_free_blocks() == 2 and a.num_allocated_blocks(2) == 0 and mapping == {7: 0}
+    a.swap_in(2, [7, 8, 9, 8], mapping)     # fits: two fresh blocks, block 8 taken once
+    assert a.get_num_free_blocks() == 0 and a.num_allocated_blocks(2) == 4
+    assert mapping[8] != mapping[9] and set(mapping) == {7, 8, 9}
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_decode_batch_kept_across_steps_equals_the_rebuilt_one(seed):
+    """Random life of a running batch -- sequences join with some context, decode token by token (new blocks,
+    copy-on-write of a forked last block), leave, rejoin -- with the index vectors updated in place; after
+    every step they equal what the step-by-step rebuild (BatchInfoBuilder, itself checked against the
+    restatement of batch_info.rs above) gives for the same sequences."""
+    rng = np.random.default_rng(300 + seed)
+    bs = 16
+    a = paged.BlockAllocator(bs, 4096)
+    db = paged.DecodeBatch(bs, 1 << 16)
+    toks, order, next_id = {}, [], 1
+
+    def join(n):
+        nonlocal next_id
+        sid, next_id = next_id, next_id + 1
+        toks[sid] = rng.integers(0, 32000, size=n).tolist()
+        a.alloc_seq(sid, n)
+        db.add(a, sid, toks[sid][-1], n)
+        order.append(sid)
+        return sid
+
+    for _ in range(int(rng.integers(1, 6))):
+        join(int(rng.integers(1, 300)))
+    for step in range(60):
+        ev = rng.random()
+        if ev < 0.15 and len(order) < 12:
+            join(int(rng.choice([1, 15, 16, 17, int(rng.integers(1, 2000))])))
+        elif ev < 0.25 and len(order) > 1:
+            sid = order.pop(int(rng.integers(len(order))))
+            db.remove(sid)
+            a.delete(sid)
+        elif ev < 0.35 and order:
+            # fork a sequence (blocks shared) and let the child join: its next token must copy the last block
+            src = order[int(rng.integers(len(order)))]
+            sid, next_id = next_id, next_id + 1
+            toks[sid] = list(toks[src])
+            a.copy(src, sid, len(toks[src]))
+            db.add(a, sid, toks[sid][-1], len(toks[sid]))
+            order.append(sid)
+        # one generation step for everybody, row by row or all rows in one call
+        new = rng.integers(0, 32000, size=len(order)).tolist()
+        for sid, t in zip(order, new):
+            n0 = len(toks[sid])
+            toks[sid].append(t)
+            a.append_slots(sid, n0, n0 + 1)
+            if step % 2 == 0:
+                db.advance(a, sid, t)
+        if step % 2 == 1:
+            db.advance_all(a, new)
+        assert len(db) == len(order)
+        b = paged.BatchInfoBuilder(bs, 1 << 16, 1)
+        for sid in order:
+            b.sched_out(a, sid, toks[sid], len(toks[sid]) - 1)
+        assert _as_dict(db.info()) == _as_dict(b.finish())
+    with pytest.raises(HipAttnError, match="not in the batch"):
+        db.advance(a, 99999, 1)
+    with pytest.raises(HipAttnError, match="in the batch already"):
+        db.add(a, order[0], 1, len(toks[order[0]]))
+
+
+def test_step_generation_hand_case():
+    """8 blocks of 4 tokens.  Sequences 1, 2, 3 (arrival order) hold 3 + 3 + 2 = 8 blocks, all full: nothing is
+    free.  Serving 1 needs a free block, so the latest arrival (3) is preempted and releases 2; 1 takes one
+    (block 7, the one freed last... the free list is a stack), 2 takes the other; nobody is left for 3."""
+    a = paged.BlockAllocator(4, 8)
+    a.alloc_seq(1, 12)
+    a.alloc_seq(2, 12)
+    a.alloc_seq(3, 8)
+    assert a.get_num_free_blocks() == 0
+    scheduled, preempted, copies = a.step_generation([1, 2, 3], [13, 13, 9], [12, 12, 8])
+    assert (scheduled, preempted, copies) == ([1, 2], [3], [])
+    assert a.num_allocated_blocks(1) == 4 and a.num_allocated_blocks(2) == 4 and a.num_allocated_blocks(3) == 0
+    assert a.get_num_free_blocks() == 0
+    # trim(3, 0) released blocks 6 then 7; the stack hands 7 to sequence 1 and 6 to sequence 2
+    assert a.get_block_idxes(1, 13)[-1] == 7 * 4 and a.get_block_idxes(2, 13)[-1] == 6 * 4
+    # next step: again nothing free; 2 is preempted for 1, and 1 -- one free block is all the check asks for,
+    # needed or not -- goes on
+    scheduled, preempted, _ = a.step_generation([1, 2], [14, 14], [13, 13])
+    assert (scheduled, preempted) == ([1], [2]) and a.get_num_free_blocks() == 4
+    # a lone sequence that finds nothing free preempts itself
+    b = paged.BlockAllocator(4, 2)
+    b.alloc_seq(5, 8)
+    assert b.step_generation([5], [9], [8]) == ([], [5], [])
+    assert b.get_num_free_blocks() == 2
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_step_generation_matches_restatement(seed):
+    rng = np.random.default_rng(400 + seed)
+    bs, nb = 8, 40
+    a, r = paged.BlockAllocator(bs, nb), ref.BlockAllocator(bs, nb)
+    lens, running, next_id = {}, [], 1
+    for step in range(80):
+        # admit while the policy allows (by arrival: ids grow)
+        while rng.random() < 0.5:
+            n = int(rng.integers(1, 60))
+            assert a.can_allocate(n) == r.can_allocate(n)
+            if not a.can_allocate(n):
+                break
+            a.alloc_seq(next_id, n)
+            r.alloc_seq(next_id, n)
+            lens[next_id] = n
+            running.append(next_id)
+            next_id += 1
+        if rng.random() < 0.1 and running:   # a fork: shared blocks, copy-on-write on the next append
+            src = running[int(rng.integers(len(running)))]
+            a.copy(src, next_id, lens[src])
+            r.copy(src, next_id, lens[src])
+            lens[next_id] = lens[src]
+            running.append(next_id)
+            next_id += 1
+        if rng.random() < 0.1 and running:
+            sid = running.pop(int(rng.integers(len(running))))
+            a.delete(sid)
+            r.delete(sid)
+        grow = [1 for _ in running]   # a generation step: one token, hence at most one block, per sequence
+        args = ([s for s in running], [lens[s] + g for s, g in zip(running, grow)], [lens[s] for s in running])
+        got = a.step_generation(*args)
+        want = ref.step_generation(r, list(zip(*args)))
+        assert got == (want[0], want[1], want[2])
+        for s, g in zip(running, grow):
+            if s in got[0]:
+                lens[s] += g
+        running = [s for s in running if s in got[0]]
+        assert a.get_num_free_blocks() == r.get_num_free_blocks()
+        for s in running:
+            assert a.get_block_idxes(s, lens[s]).tolist() == r.get_block_idxes(s, lens[s])
