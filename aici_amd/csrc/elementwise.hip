@@ -271,13 +271,14 @@ template <typename T, int MODE /*0 = f32 bias rows, 1 = packed allow-bits*/>
 __global__ __launch_bounds__(1024) void bias_argmax_kernel(const T *__restrict__ logits, int64_t logit_stride,
                                                            const float *__restrict__ bias, int64_t bias_stride,
                                                            const uint8_t *__restrict__ mask, int64_t mask_stride,
-                                                           int64_t mask_bytes, const int32_t *__restrict__ rows,
+                                                           int64_t mask_bytes, const int32_t *__restrict__ rows, int64_t nrows,
                                                            int vocab, int32_t *__restrict__ out_tokens,
                                                            float *__restrict__ out_logits) {
   __shared__ float s_val[16];
   __shared__ int s_idx[16];
   const int64_t seq = blockIdx.x;
-  const int64_t row = rows ? (int64_t)rows[seq] : seq;
+  int64_t row = rows ? (int64_t)rows[seq] : seq;
+  row = row < 0 ? 0 : (row >= nrows ? nrows - 1 : row);  // a bad row index reads a wrong row, never outside
   const T *lg = logits + seq * logit_stride;
   float best = -INFINITY;
   int best_i = 0x7fffffff;
@@ -334,7 +335,7 @@ template <typename T, int MODE>
 __global__ __launch_bounds__(256) void bias_argmax_slice_kernel(const T *__restrict__ logits, int64_t logit_stride,
                                                                 const float *__restrict__ bias, int64_t bias_stride,
                                                                 const uint8_t *__restrict__ mask, int64_t mask_stride,
-                                                                int64_t mask_bytes, const int32_t *__restrict__ rows,
+                                                                int64_t mask_bytes, const int32_t *__restrict__ rows, int64_t nrows,
                                                                 int vocab, int per_slice /* multiple of 8 */,
                                                                 float *__restrict__ part_val,
                                                                 int32_t *__restrict__ part_idx) {
@@ -342,7 +343,8 @@ __global__ __launch_bounds__(256) void bias_argmax_slice_kernel(const T *__restr
   __shared__ int s_idx[4];
   const int64_t seq = blockIdx.y;
   const int slice = blockIdx.x;
-  const int64_t row = rows ? (int64_t)rows[seq] : seq;
+  int64_t row = rows ? (int64_t)rows[seq] : seq;
+  row = row < 0 ? 0 : (row >= nrows ? nrows - 1 : row);  // a bad row index reads a wrong row, never outside
   const T *lg = logits + seq * logit_stride;
   const int begin = slice * per_slice;
   const int end = min(begin + per_slice, vocab);
@@ -691,11 +693,11 @@ void bias_argmax_impl(const hipattn_tensor *logits, const hipattn_tensor *bias, 
   if (bias)                                                                                                     \
     bias_argmax_slice_kernel<TT, 0><<<grid, 256, 0, stream>>>(                                                   \
         static_cast<const TT *>(logits->data), logits->strides[0], static_cast<const float *>(bias->data),      \
-        bias->strides[0], nullptr, 0, 0, rp, (int)V, per_slice, pv, pi);                                        \
+        bias->strides[0], nullptr, 0, 0, rp, nrows, (int)V, per_slice, pv, pi);                                        \
   else                                                                                                          \
     bias_argmax_slice_kernel<TT, 1><<<grid, 256, 0, stream>>>(                                                   \
         static_cast<const TT *>(logits->data), logits->strides[0], nullptr, 0,                                  \
-        static_cast<const uint8_t *>(mask->data), mask->strides[0], mask->sizes[1], rp, (int)V, per_slice, pv, pi)
+        static_cast<const uint8_t *>(mask->data), mask->strides[0], mask->sizes[1], rp, nrows, (int)V, per_slice, pv, pi)
     if (logits->dtype == HIPATTN_F16) {
       HA_BAW(half_t);
     } else {
@@ -712,11 +714,11 @@ void bias_argmax_impl(const hipattn_tensor *logits, const hipattn_tensor *bias, 
   if (bias)                                                                                                     \
     bias_argmax_kernel<TT, 0><<<dim3((unsigned)S), threads, 0, stream>>>(                                        \
         static_cast<const TT *>(logits->data), logits->strides[0], static_cast<const float *>(bias->data),      \
-        bias->strides[0], nullptr, 0, 0, rp, (int)V, static_cast<int32_t *>(out_tokens->data), ol);             \
+        bias->strides[0], nullptr, 0, 0, rp, nrows, (int)V, static_cast<int32_t *>(out_tokens->data), ol);             \
   else                                                                                                          \
     bias_argmax_kernel<TT, 1><<<dim3((unsigned)S), threads, 0, stream>>>(                                        \
         static_cast<const TT *>(logits->data), logits->strides[0], nullptr, 0,                                  \
-        static_cast<const uint8_t *>(mask->data), mask->strides[0], mask->sizes[1], rp, (int)V,                 \
+        static_cast<const uint8_t *>(mask->data), mask->strides[0], mask->sizes[1], rp, nrows, (int)V,                 \
         static_cast<int32_t *>(out_tokens->data), ol)
   switch (logits->dtype) {
     case HIPATTN_F32: HA_BA(float); break;

@@ -271,6 +271,20 @@ def bias_argmax(logits: torch.Tensor, bias: Optional[torch.Tensor] = None, mask:
     return (tokens, best) if return_logits else tokens
 
 
+def bias_sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, uniforms: torch.Tensor,
+                bias: Optional[torch.Tensor] = None, mask: Optional[torch.Tensor] = None,
+                bias_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """AICI bias, temperature, top-p and the draw (tmodel.rs:277-283, 172-194, 236-268) for every row at once.
+    temperature / top_p / uniforms: f32 [S]; rows with temperature < 1e-5 are greedy; uniforms in [0, 1) are
+    the caller's random numbers (one per row).  Returns int32 [S]."""
+    S = logits.size(0)
+    tokens = torch.empty((S,), dtype=torch.int32, device=logits.device)
+    call("hipattn_bias_sample", _desc(logits, "logits"), _desc(bias, "bias"), _desc(mask, "mask"),
+         _desc(bias_rows, "bias_rows"), _desc(temperature, "temperature"), _desc(top_p, "top_p"),
+         _desc(uniforms, "uniforms"), _desc(tokens, "out_tokens"), _stream(logits))
+    return tokens
+
+
 def stream_probe(mode: str, dst: Optional[torch.Tensor], src: Optional[torch.Tensor],
                  chunks: Optional[torch.Tensor] = None) -> None:
     """One launch of the library's memory-system yardstick: "read" src once, "copy" src to dst, "fill"

@@ -149,3 +149,11 @@ def aici_greedy(logits: torch.Tensor, allow_masks: torch.Tensor) -> torch.Tensor
     as a 0/-inf bias and the arg-max taken (tmodel.rs:277-283, 234-236), all rows in one
     launch and without materialising f32 bias rows.  Returns int32 [S]."""
     return kernels.bias_argmax(logits, mask=allow_masks)
+
+
+def aici_sample(logits: torch.Tensor, allow_masks: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
+                uniforms: torch.Tensor) -> torch.Tensor:
+    """The sampling half with temperature and top-p (tmodel.rs:172-194, 236-268) under the same packed
+    allow-masks: rows with temperature < 1e-5 are greedy, the others are drawn with the caller's uniform
+    numbers (one per row, in [0, 1)).  All rows in one launch, no host round trip.  Returns int32 [S]."""
+    return kernels.bias_sample(logits, temperature, top_p, uniforms, mask=allow_masks)

@@ -230,6 +230,12 @@ def streaming_leg(dev, stream, steps: int) -> dict:
     allowed = W.allow_mask(5, S, V)
     mask = torch.from_numpy(np.packbits(np.pad(allowed, ((0, 0), (0, (-V) % 32))), axis=1, bitorder="little")).to(dev)
     run("bias_argmax 128 x 128256, packed allow-bits", lambda: K.bias_argmax(lg, mask=mask), S * V * 2 + mask.numel())
+    temp = torch.full((S,), 0.8, device=dev)
+    u = torch.rand((S,), device=dev)
+    for tp in (1.0, 0.9):
+        top_p = torch.full((S,), tp, device=dev)
+        run(f"bias_sample 128 x 128256, packed allow-bits, temperature 0.8, top_p {tp} (algorithmic bytes: one pass)",
+            lambda: K.bias_sample(lg, temp, top_p, u, mask=mask), S * V * 2 + mask.numel())
     row = (V + 1000) & ~63
     bias = torch.full((S, row), float("-inf"), dtype=torch.float32, device=dev)
     bias[:, :V][torch.from_numpy(allowed).to(dev)] = 0.0

@@ -164,6 +164,119 @@ def test_bias_argmax_bias_rows_and_packed_mask(device, dtype):
         K.bias_argmax(ld)
 
 
+def _sample_check(logits, bias, temperature, top_p, u, got):
+    """Row by row against the oracle.  The oracle's token is expected; where the two differ the draw must sit
+    on an edge: u * total within 1e-5 (relative) of the cumulative weight that separates the two tokens, or
+    the nucleus cut within f32 rounding of admitting one more token.  Returns the number of rows that differ."""
+    differ = 0
+    V = logits.shape[1]
+    for s in range(logits.shape[0]):
+        want = aici.sample(logits[s], bias[s], float(temperature[s]), float(top_p[s]), float(u[s]))
+        t = int(got[s])
+        if t == want:
+            continue
+        differ += 1
+        assert temperature[s] >= aici.SAMPLING_EPS, (s, t, want)      # the arg-max is exact
+        prs = torch.softmax((logits[s].float() + bias[s][:V]).double() / float(temperature[s]), 0).numpy()
+        w = prs.copy()
+        if 0.0 < top_p[s] < 1.0:
+            order = sorted(range(V), key=lambda i: (-prs[i], i))
+            mass, kept = 0.0, np.zeros(V, dtype=bool)
+            for i in order:
+                if mass >= float(top_p[s]) * (1 + 1e-5):
+                    break
+                kept[i] = True
+                mass += prs[i]
+            w = np.where(kept, prs, 0.0)
+        assert w[t] > 0, (s, t, want)
+        cum = np.cumsum(w)
+        c = float(u[s])
+        lo, hi = (cum[t - 1] if t else 0.0) / cum[-1], cum[t] / cum[-1]
+        assert lo - 1e-4 <= c <= hi + 1e-4, (s, t, want, lo, c, hi)
+    return differ
+
+
+@pytest.mark.parametrize("dtype,V,mode", [(torch.bfloat16, 128256, "mask"), (torch.float16, 50000, "bias"),
+                                          (torch.float32, 1000, "bias"), (torch.bfloat16, 4097, "mask")])
+def test_bias_sample_matches_the_oracle(device, dtype, V, mode):
+    """Temperature + top-p sampling under the AICI bias against the restatement of tmodel.rs:172-194,
+    236-268, row by row with the caller's uniform numbers: greedy rows, plain sampling (top_p 0 and 1),
+    nuclei from tiny to almost everything, sharp and flat temperatures."""
+    S = 40
+    g = torch.Generator().manual_seed(11)
+    rng = np.random.default_rng(11)
+    logits = (torch.randn((S, V), generator=g) * 2.5).to(dtype)
+    allowed = W.allow_mask(6, S, V, 0.05 if V > 5000 else 0.5)
+    allowed[:, 17] = True
+    packed = np.stack([aici.pack_allowed(a) for a in allowed])
+    bias = torch.from_numpy(np.stack([aici.apply_to_slice_fast(p, aici.bias_row_len(V)) for p in packed]))
+    temperature = torch.tensor(rng.choice([0.0, 1e-6, 0.05, 0.5, 0.8, 1.0, 1.7, 10.0], size=S), dtype=torch.float32)
+    top_p = torch.tensor(rng.choice([0.0, 1.0, 1e-4, 0.1, 0.5, 0.9, 0.95, 0.999], size=S), dtype=torch.float32)
+    u = torch.tensor(rng.random(S), dtype=torch.float32)
+    u[0], u[1] = 0.0, 0.99999994
+    kw = dict(mask=torch.from_numpy(packed).to(device)) if mode == "mask" else dict(bias=bias.to(device))
+    got = K.bias_sample(logits.to(device), temperature.to(device), top_p.to(device), u.to(device), **kw).cpu()
+    assert allowed[np.arange(S), got.numpy()].all()           # never a disallowed token
+    differ = _sample_check(logits, bias, temperature, top_p, u, got)
+    assert differ <= 2, differ
+    # the launch is a function of its inputs: same tokens again
+    again = K.bias_sample(logits.to(device), temperature.to(device), top_p.to(device), u.to(device), **kw).cpu()
+    assert torch.equal(got, again)
+
+
+def test_bias_sample_equal_values_and_distribution(device):
+    """Coarse logits (many equal probabilities, the usual case with 16-bit logits): one row drawn with 4096
+    evenly spaced uniform numbers.  The nucleus cut must split a run of equal values by ascending id, and the
+    draws must reproduce the kept weights as frequencies."""
+    V, n = 3000, 4096
+    g = torch.Generator().manual_seed(12)
+    row = (torch.randn((V,), generator=g) * 1.5).mul(2).round().div(2).to(torch.bfloat16)   # steps of 0.5
+    logits = row[None].expand(n, V).contiguous()
+    bias = torch.zeros((1, aici.bias_row_len(V)))
+    bias[0, 5::7] = float("-inf")
+    rows = torch.zeros((n,), dtype=torch.int32)
+    u = ((torch.arange(n) + 0.5) / n).float()
+    for top_p in (0.3, 0.62, 0.9, 1.0):
+        temperature = torch.full((n,), 0.7)
+        got = K.bias_sample(logits.to(device), temperature.to(device), torch.full((n,), top_p).to(device),
+                            u.to(device), bias=bias.to(device), bias_rows=rows.to(device)).cpu().numpy()
+        prs = torch.softmax((row.float() + bias[0, :V]) / 0.7, 0).numpy()
+        w = aici.nucleus_weights(prs, top_p) if top_p < 1.0 else prs
+        kept = w > 0
+        # the kept set: everything above the cut, and of the values equal to the cut the lowest ids
+        cut = prs[kept].min()
+        assert np.array_equal(kept, (prs > cut) | ((prs == cut) & (np.cumsum(prs == cut) <= (kept & (prs == cut)).sum())))
+        assert kept[got].all()
+        freq = np.bincount(got, minlength=V) / n
+        assert np.abs(freq - w / w.sum()).max() <= 1.01 / n + 1e-6
+        # draw by draw: the oracle's token, except where u sits on an edge between two tokens -- the
+        # cumulative weights are f32 sums formed in different orders on the two sides (3000 terms: 1e-5)
+        want = np.array([aici.weighted_index(w, float(x)) for x in u])
+        off = np.nonzero(got != want)[0]
+        assert len(off) <= n // 100, len(off)
+        cum = np.cumsum(w.astype(np.float64)) / w.astype(np.float64).sum()
+        for i in off:
+            t = int(got[i])
+            assert (cum[t - 1] if t else 0.0) - 1e-4 <= float(u[i]) <= cum[t] + 1e-4, (top_p, i, t, int(want[i]))
+
+
+def test_bias_sample_argument_errors(device):
+    lg = torch.zeros((2, 64), dtype=torch.float16, device=device)
+    f = lambda *v: torch.tensor(v, dtype=torch.float32, device=device)
+    m = torch.full((2, 8), 255, dtype=torch.uint8, device=device)
+    assert K.bias_sample(lg, f(1.0, 0.0), f(1.0, 1.0), f(0.5, 0.5), mask=m).tolist() == [32, 0]
+    with pytest.raises(HipAttnError, match="exactly one"):
+        K.bias_sample(lg, f(1.0, 1.0), f(1.0, 1.0), f(0.5, 0.5))
+    with pytest.raises(HipAttnError, match=r"top_p must be f32 \[S\]"):
+        K.bias_sample(lg, f(1.0, 1.0), f(1.0), f(0.5, 0.5), mask=m)
+    none = torch.zeros((2, 8), dtype=torch.uint8, device=device)
+    assert K.bias_sample(lg, f(1.0, 1.0), f(0.9, 1.0), f(0.5, 0.5), mask=none).tolist() == [0, 0]   # nothing allowed
+    # a bias row index outside the rows given reads the nearest row, never beyond
+    far = torch.tensor([5, -3], dtype=torch.int32, device=device)
+    assert K.bias_sample(lg, f(0.0, 0.0), f(1.0, 1.0), f(0.5, 0.5), mask=m, bias_rows=far).tolist() == [0, 0]
+    assert K.bias_argmax(lg, mask=m, bias_rows=far).tolist() == [0, 0]
+
+
 def test_streams_events_and_memory_figures(device):
     props = K.cuda_get_device_properties(0)
     assert props.multi_processor_count == 256 and props.total_memory > 200 * 2 ** 30

@@ -150,3 +150,72 @@ def test_aici_mask_bit_order_and_bias():
     assert tok.item() == 69
     logits[0, 9] = 1000.0
     assert aici.biased_argmax(logits, torch.from_numpy(row).reshape(1, -1)).item() == 9
+
+
+# ---- sampling (tmodel.rs:172-194, 236-268): pinned by what the procedure reduces to in special cases -------
+
+def test_nucleus_weights_hand_case_and_brute_force():
+    # sorted: 0.4 (id 2), 0.3 (id 0), 0.2 (id 3), 0.1 (id 1).  top_p 0.65: 0.4 kept (before: 0), 0.3 kept
+    # (before: 0.4 < 0.65), 0.2 dropped (before: 0.7 >= 0.65)
+    prs = np.array([0.3, 0.1, 0.4, 0.2], dtype=np.float32)
+    assert aici.nucleus_weights(prs, 0.65).tolist() == [np.float32(0.3), 0.0, np.float32(0.4), 0.0]
+    # a token is kept exactly when the mass before it is below top_p: 0.7 itself keeps the third
+    assert np.count_nonzero(aici.nucleus_weights(prs, 0.7000001)) == 3
+    # equal values: the stable sort takes the lower ids first
+    tie = np.array([0.25, 0.25, 0.25, 0.25], dtype=np.float32)
+    assert aici.nucleus_weights(tie, 0.5).tolist() == [0.25, 0.25, 0.0, 0.0]
+    assert aici.nucleus_weights(tie, 0.51).tolist() == [0.25, 0.25, 0.25, 0.0]
+    # brute force on random small distributions: the kept set is the shortest prefix of the sorted order
+    # whose mass reaches top_p
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        n = int(rng.integers(2, 12))
+        p = rng.random(n).astype(np.float32)
+        p /= p.sum()
+        top_p = float(rng.uniform(0.05, 0.95))
+        kept = aici.nucleus_weights(p, top_p)
+        order = sorted(range(n), key=lambda i: (-p[i], i))
+        want, mass = np.zeros(n, dtype=np.float32), np.float32(0.0)
+        for i in order:
+            if mass >= np.float32(top_p):
+                break
+            want[i] = p[i]
+            mass = np.float32(mass + p[i])
+        assert np.array_equal(kept, want)
+
+
+def test_weighted_index_is_the_inverse_cdf():
+    w = np.array([0.0, 2.0, 0.0, 1.0, 1.0], dtype=np.float32)   # cumulative 0 2 2 3 4
+    assert [aici.weighted_index(w, u) for u in (0.0, 0.49, 0.5, 0.74, 0.75, 0.999)] == [1, 1, 3, 3, 4, 4]
+    # a zero weight is never drawn, whatever u
+    assert all(aici.weighted_index(w, u) in (1, 3, 4) for u in np.linspace(0, 0.9999, 1000))
+    # frequencies over an even grid of u follow the weights
+    p = np.array([0.1, 0.2, 0.3, 0.4], dtype=np.float32)
+    draws = np.array([aici.weighted_index(p, u) for u in (np.arange(10000) + 0.5) / 10000])
+    assert np.allclose(np.bincount(draws, minlength=4) / 10000, p, atol=2e-4)
+
+
+def test_sample_reduces_to_known_procedures():
+    g = torch.Generator().manual_seed(3)
+    V = 500
+    logits = torch.randn((V,), generator=g) * 3
+    bias = torch.zeros((aici.bias_row_len(V),))
+    bias[::3] = float("-inf")
+    allowed = torch.isfinite(bias[:V])
+    greedy = int((logits + bias[:V]).argmax())
+    # temperature below SAMPLING_EPS is the arg-max; a sharp temperature or a tiny nucleus gives it too
+    assert aici.sample(logits, bias, 0.0, 0.9, 0.37) == greedy
+    assert all(aici.sample(logits, bias, 1e-3, 1.0, u) == greedy for u in (0.0, 0.5, 0.999))
+    assert all(aici.sample(logits, bias, 1.0, 1e-6, u) == greedy for u in (0.0, 0.5, 0.999))
+    # top_p = 1 (or 0): plain sampling -- over an even grid of u the frequencies are the softmax, and no
+    # disallowed token is ever drawn
+    p = torch.softmax((logits + bias[:V]) / 0.8, 0).numpy()
+    n = 20000
+    draws = np.array([aici.sample(logits, bias, 0.8, 1.0, u) for u in (np.arange(n) + 0.5) / n])
+    assert allowed[draws].all()
+    assert np.abs(np.bincount(draws, minlength=V) / n - p).max() < 1.5 / n + 1e-6
+    # with a nucleus the draws stay inside the kept set and follow its renormalised weights
+    kept = aici.nucleus_weights(p, 0.6)
+    draws = np.array([aici.sample(logits, bias, 0.8, 0.6, u) for u in (np.arange(n) + 0.5) / n])
+    assert (kept[draws] > 0).all() and 0.6 <= kept.sum() < 0.6 + p.max()
+    assert np.abs(np.bincount(draws, minlength=V) / n - kept / kept.sum()).max() < 1.5 / n + 1e-6
