@@ -505,12 +505,15 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void paged_decode_flat_kern
   __shared__ int s_ctx[kFlatMaxSeqs];
   __shared__ int s_excl[kFlatMaxSeqs + 1];  // block pairs before sequence s; [S] = all
   __shared__ int s_wsum[4];
+  __shared__ f32x4_t s_park[4][NDT][64];  // a wavefront's partial result waiting to be written (see below)
+  __shared__ float s_park_ml[4][2][64];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int kg = lane >> 4;
   const int col = lane & 15;
   const int S = p.num_seqs;
+  bool parked = false;
 
   // Exclusive prefix of the pair counts, thread t owning sequences 4t..4t+3.
   {
@@ -660,19 +663,39 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void paged_decode_flat_kern
           for (int i = 0; i < 4; i++) rr[i] = from_float<T>(acc[dt][i] * inv);
           *reinterpret_cast<u32x2_t *>(op + dt * 16) = *reinterpret_cast<u32x2_t *>(rr);
         }
-      } else {
-        const int64_t pidx = (int64_t)(2 * w + (u != u_first ? 1 : 0)) * p.flat_cols + col;
-        float *ap = p.ws_acc + pidx * HD + kg * 4;
+      } else if (u == u_first && u + n < u_end) {
+          // The piece at the head of the range, with more of the range to stream after it: parked in LDS and
+          // written out after the loop.  A store issued here would sit in the same in-order counter as the
+          // loads that follow, and the first wait for those loads would also wait for the store to be
+          // acknowledged (measured: 6.6 us of a 126 us step).
 #pragma unroll
-        for (int dt = 0; dt < NDT; dt++) *reinterpret_cast<f32x4_t *>(ap + dt * 16) = acc[dt];
-        if (kg == 0) {
-          p.ws_m[pidx] = m_run;
-          p.ws_l[pidx] = l_tot;
+          for (int dt = 0; dt < NDT; dt++) s_park[wave][dt][lane] = acc[dt];
+          s_park_ml[wave][0][lane] = m_run;
+          s_park_ml[wave][1][lane] = l_tot;
+          parked = true;
+        } else {
+          const int64_t pidx = (int64_t)(2 * w + (u != u_first ? 1 : 0)) * p.flat_cols + col;
+          float *ap = p.ws_acc + pidx * HD + kg * 4;
+#pragma unroll
+          for (int dt = 0; dt < NDT; dt++) *reinterpret_cast<f32x4_t *>(ap + dt * 16) = acc[dt];
+          if (kg == 0) {
+            p.ws_m[pidx] = m_run;
+            p.ws_l[pidx] = l_tot;
+          }
         }
-      }
     }
     u += n;
     if (pr0 + n == pairs && h == hk - 1) seq++;
+  }
+  if (parked) {  // only lanes that hold a query head parked anything (slot 2w: the piece began the range)
+    const int64_t pidx = (int64_t)(2 * w) * p.flat_cols + col;
+    float *ap = p.ws_acc + pidx * HD + kg * 4;
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++) *reinterpret_cast<f32x4_t *>(ap + dt * 16) = s_park[wave][dt][lane];
+    if (kg == 0) {
+      p.ws_m[pidx] = s_park_ml[wave][0][lane];
+      p.ws_l[pidx] = s_park_ml[wave][1][lane];
+    }
   }
 }
 

@@ -62,6 +62,7 @@ Tuning tuning_from_env() {
   t.prefill_kernel = env_int("HIPATTN_PREFILL_KERNEL", 0);
   t.paged_prefill_dma = env_int("HIPATTN_PAGED_PREFILL_DMA", -1);
   t.cache_move_lds = env_int("HIPATTN_CACHE_MOVE_LDS", -1);
+  t.prefill_wg_heads = env_int("HIPATTN_PREFILL_WG_HEADS", 0);
   t.prefill_rescale_log2 = env_int("HIPATTN_PREFILL_RESCALE_LOG2", 8);
   if (t.prefill_rescale_log2 < 0 || t.prefill_rescale_log2 > 16) t.prefill_rescale_log2 = 8;
   return t;
@@ -80,6 +81,7 @@ const TuningField kTuningFields[] = {
     {"prefill_kernel", &Tuning::prefill_kernel, 0, 3},
     {"paged_prefill_dma", &Tuning::paged_prefill_dma, -1, 1},
     {"cache_move_lds", &Tuning::cache_move_lds, -1, 1},
+    {"prefill_wg_heads", &Tuning::prefill_wg_heads, 0, 8},
     {"prefill_rescale_log2", &Tuning::prefill_rescale_log2, 0, 16},
 };
 }  // namespace

@@ -425,7 +425,9 @@ char *hipattn_shutdown(void);
  * call, else 2..64), prefill_kernel (0 library's choice, 1 eight wavefronts,
  * 2 / 3 four wavefronts with 2 / 1 row tiles), paged_prefill_dma (-1 library's
  * choice, 0 staged tiles), cache_move_lds (-1 library's choice, 0 never the
- * LDS-transposing kernels), prefill_rescale_log2 (0..16, default 8: the prefill
+ * LDS-transposing kernels), prefill_wg_heads (query heads of one kv group per
+ * workgroup of the eight-wavefront prefill kernel, at most; 0 and 1: one),
+ * prefill_rescale_log2 (0..16, default 8: the prefill
  * kernels move a row's reference maximum only when the row outgrows it by
  * more than 2^value; 0 follows the row maximum exactly, as the reference
  * does).  Every setting computes the same results, prefill_rescale_log2 up to

@@ -271,3 +271,26 @@ def test_sliding_window_closed_forms_and_large_launch(device):
     ones = torch.ones_like(dv.v)
     c = K.flash_attn_varlen(dv.q, dv.k, ones, dv.cu_q, dv.cu_k, p.max_q, p.max_k, p.scale, False, window=(127, 0))
     assert (c.float().cpu() - 1.0).abs().max().item() <= 2 ** -7
+
+
+@pytest.mark.parametrize("limit", [2, 4, 8])
+def test_several_heads_of_a_kv_group_per_workgroup(device, tuning, limit):
+    """The eight-wavefront kernel can give a workgroup 2, 4 or 8 query heads of one kv group (and 128, 64 or 32
+    rows of each) instead of 256 rows of one head: same results, to the bit, as one head per workgroup -- the
+    arithmetic of a row does not depend on which wavefront runs it -- for GQA ratios 4 and 8, ragged chunks with
+    prior context, the log-sum-exp and the fp32 output."""
+    for seed, (Hq, Hkv, d, dtype) in [(51, (32, 8, 128, torch.bfloat16)), (52, (16, 2, 64, torch.float16))]:
+        p = general_inputs(seed, [300, 1, 70, 513], [300, 40, 517, 513], Hq, Hkv, d, dtype)
+        dv = p.to(device)
+        args = (dv.q, dv.k, dv.v, dv.cu_q, dv.cu_k, p.max_q, p.max_k, p.scale, True)
+        tuning("prefill_kernel", 1)
+        tuning("prefill_wg_heads", 1)
+        want, want_lse = K.flash_attn_varlen(*args, return_lse=True)
+        want32 = K.flash_attn_varlen(*args, out_dtype=torch.float32)
+        tuning("prefill_wg_heads", limit)
+        got, got_lse = K.flash_attn_varlen(*args, return_lse=True)
+        got32 = K.flash_attn_varlen(*args, out_dtype=torch.float32)
+        assert torch.equal(got, want) and torch.equal(got32, want32)
+        for b, lq in enumerate(p.lens_q):   # rows past a sequence's length are not written
+            assert torch.equal(got_lse[b, :, :lq], want_lse[b, :, :lq])
+        assert (got.cpu().double() - fp64(p)).abs().max().item() <= TOL[dtype]
