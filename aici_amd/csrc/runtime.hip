@@ -111,11 +111,12 @@ void *library_workspace(WorkspaceUser user, size_t bytes, hipStream_t stream) {
   want = (want + 255) & ~(size_t)255;
   void *fresh = nullptr;
   HA_HIP(hipMalloc(&fresh, want));
-  // Counters kept in the buffer start at zero.  A blocking fill: nothing else is ordered against it.
-  hipError_t e = hipMemset(fresh, 0, want);
+  // Counters kept in the buffer start at zero.  The fill goes onto the stream that the buffer belongs to (which is
+  // not being captured here), ahead of the kernels that use it.
+  hipError_t e = hipMemsetAsync(fresh, 0, want, stream);
   if (e != hipSuccess) {
     (void)hipFree(fresh);
-    fail("hipMemset of a new scratch buffer failed: %s", hipGetErrorString(e));
+    fail("clearing a new scratch buffer failed: %s", hipGetErrorString(e));
   }
   if (ws.ptr != nullptr) g_retired.emplace_back(dev, ws.ptr);
   ws.ptr = fresh;

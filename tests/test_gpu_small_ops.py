@@ -164,6 +164,32 @@ def test_bias_argmax_bias_rows_and_packed_mask(device, dtype):
         K.bias_argmax(ld)
 
 
+def test_bias_argmax_wide_rows_call_after_call(device):
+    """Long 16-bit rows are cut into slices whose winners meet in a per-row key and counter kept between calls:
+    call after call with changing row counts, negative and infinite winners, and the winning value itself."""
+    g = torch.Generator().manual_seed(11)
+    V = 65536
+    for S in (128, 5, 64, 1):
+        logits = (torch.randn((S, V), generator=g) - 6.0).to(torch.bfloat16)      # every value negative
+        logits[0, 4242] = float("-inf")
+        allowed = torch.rand((S, V), generator=g) < 0.03
+        if S > 2:
+            allowed[2, :] = False
+            allowed[2, 77] = True                                                  # one token, wherever its value lies
+        packed = torch.from_numpy(np.stack([aici.pack_allowed(a) for a in allowed.numpy()]))
+        masked = torch.where(allowed, logits.float(), torch.tensor(float("-inf")))
+        want = masked.argmax(dim=1)
+        for _ in range(3):
+            tok, best = K.bias_argmax(logits.to(device), mask=packed.to(device), return_logits=True)
+            assert torch.equal(tok.cpu().long(), want)
+            assert torch.equal(best.cpu(), masked[torch.arange(S), want])
+    pos_inf = torch.zeros((2, V), dtype=torch.float16, device=device)
+    pos_inf[1, 40000] = float("inf")
+    tok, best = K.bias_argmax(pos_inf, mask=torch.full((2, V // 8), 255, dtype=torch.uint8, device=device),
+                              return_logits=True)
+    assert tok.tolist() == [0, 40000] and best.tolist() == [0.0, float("inf")]
+
+
 def _sample_check(logits, bias, temperature, top_p, u, got):
     """Row by row against the oracle.  The oracle's token is expected; where the two differ the draw must sit
     on an edge: u * total within 1e-5 (relative) of the cumulative weight that separates the two tokens, or
