@@ -448,7 +448,7 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
 // contiguous -- and reads both operands with ds_read_b128.
 // ---------------------------------------------------------------------------
 // Where the eight-wavefront kernel takes its K/V tiles from.
-enum { W8_ROWS = 0, W8_PAGED = 1, W8_PAGED_DMA = 2 };
+enum { W8_ROWS = 0, W8_PAGED = 1, W8_PAGED_DMA = 2, W8_PAGED_DMA_PART = 3 };
 
 template <int HDP>
 struct TileW8 {
@@ -465,7 +465,11 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   typedef typename Vec8<T>::type vec8;
   typedef TileW8<HDP> TL;
   constexpr bool PAGED = MODE != W8_ROWS;
-  constexpr bool DMA = MODE == W8_PAGED_DMA;
+  constexpr bool DMA = MODE == W8_PAGED_DMA || MODE == W8_PAGED_DMA_PART;
+  // W8_PAGED_DMA_PART: head sizes below HDP (Phi-2's 80 in the 96-wide instance).  An image then fills only the
+  // first d / HDP of its place in LDS; the rest is cleared once, so the contraction steps and output rows past d
+  // work on zeros.
+  constexpr bool DMA_PART = MODE == W8_PAGED_DMA_PART;
   // W8_PAGED_DMA keeps a tile as the four block images of the cache, unpadded, in four stages.
   constexpr int NST = DMA ? 4 : 3;
   constexpr int STAGE_ELEMS = DMA ? 2 * BN * HDP : TL::STAGE_ELEMS;
@@ -673,6 +677,10 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   const unsigned dma_lane = dma_v ? c * 32 + g * 16 : lane * 16;
   const char *dma_base = reinterpret_cast<const char *>(dma_v ? vp : kp);
   const int64_t dma_blk_bytes = (dma_v ? p.vc_block : p.kc_block) * (int64_t)sizeof(T);
+  // The last piece of an image that is shorter than HDP: K lanes past the image's last 16-byte run and V
+  // lanes whose row lies past d fetch nothing (what lies there belongs to the next head or block).
+  const int dma_tail = p.d - 32 * (NDMA - 1);  // head elements in the last piece, 32 when d == HDP
+  const bool dma_last_ok = !DMA_PART || (dma_v ? c < dma_tail : lane < 2 * dma_tail);
   int64_t tbl_off = 0;
   auto ids_to_offsets = [&](int blk) -> int64_t {
     const int64_t bid = blk < 0 ? 0 : (blk >= p.num_blocks ? p.num_blocks - 1 : (int64_t)blk);
@@ -690,11 +698,13 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
                :                                                                                   \
                : "s"(dst), "v"(dma_lane), "s"(src)                                                 \
                : "memory", "m0")
-    switch (i) {
-      case 0: HA_DMA_PIECE(0); break;
-      case 1: HA_DMA_PIECE(1024); break;
-      case 2: HA_DMA_PIECE(2048); break;
-      default: HA_DMA_PIECE(3072); break;
+    if (!DMA_PART || i < NDMA - 1 || dma_last_ok) {
+      switch (i) {
+        case 0: HA_DMA_PIECE(0); break;
+        case 1: HA_DMA_PIECE(1024); break;
+        case 2: HA_DMA_PIECE(2048); break;
+        default: HA_DMA_PIECE(3072); break;
+      }
     }
 #undef HA_DMA_PIECE
     if (i == NDMA - 1) {
@@ -705,6 +715,26 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   auto dma_tile = [&](int tile) {
 #pragma unroll
     for (int i = 0; i < NDMA; i++) dma_piece(tile, i);
+  };
+  // W8_PAGED_DMA_PART: clears what the images leave untouched in stages first..last: per block the K runs of
+  // head elements d..HDP and, in the last V piece, the rows d..HDP of both 8-token halves.
+  auto clear_image_tails = [&](int first, int last) {
+    if constexpr (DMA_PART) {
+      const int R = HDP - p.d;       // a multiple of 8 below 32
+      const int per_stage = 16 * R;  // 16-byte runs: 4 blocks x (2 R of K + 2 R of V)
+      for (int st = first; st <= last; st++)
+        for (int idx = tid; idx < per_stage; idx += 512) {
+          const int r = idx / (4 * R), rem = idx % (4 * R);
+          int e;
+          if (rem < 2 * R) {
+            e = r * BLK_ELEMS + (2 * p.d + rem) * 8;
+          } else {
+            const int v = rem - 2 * R;
+            e = K_ELEMS + r * BLK_ELEMS + (NDMA - 1) * 512 + ((v / R) * 32 + (32 - R) + v % R) * 8;
+          }
+          *reinterpret_cast<u32x4_t *>(smem + st * STAGE_ELEMS + e) = u32x4_t{0u, 0u, 0u, 0u};
+        }
+    }
   };
   // Waits until this wavefront's pieces of `tile` have landed (`newer`: the pieces of the tile after it
   // were issued later and may still fly), then clears the V tokens past the context in them: stale
@@ -842,11 +872,13 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     // Tile 0 flies into stage 0 while Q is turned through stages 1..3; tiles 1 and 2 follow once every
     // wavefront has its Q.
     if (n_tiles > 0) dma_tile(0);
+    clear_image_tails(0, 0);
     load_q();
     if (n_tiles > 0) dma_wait(0, false);
     __syncthreads();
     if (n_tiles > 1) dma_tile(1);
     if (n_tiles > 2) dma_tile(2);
+    clear_image_tails(1, NST - 1);  // seen by all after the barrier in front of the loop; stage 1 is first read there
   } else {
     if (n_tiles > 0) load_tile(0);
     load_q();
@@ -1136,7 +1168,7 @@ template <typename T, int HDP, int MODE = W8_ROWS>
 void launch_prefill_w8(PrefillParams p, hipStream_t stream) {
   static bool attr_set = false;  // benign race: setting twice is harmless
   auto kernel = prefill_varlen_w8_kernel<T, HDP, MODE>;
-  constexpr size_t lds_bytes = MODE == W8_PAGED_DMA ? (size_t)4 * 2 * BN * HDP * 2 : TileW8<HDP>::LDS_BYTES;
+  constexpr size_t lds_bytes = MODE >= W8_PAGED_DMA ? (size_t)4 * 2 * BN * HDP * 2 : TileW8<HDP>::LDS_BYTES;
   if (!attr_set) {
     HA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)lds_bytes));
@@ -1342,11 +1374,14 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
 template <typename T>
 void dispatch_paged(const PrefillParams &p, hipStream_t stream) {
   const int hdp = ((p.d + 31) / 32) * 32;
-  // Head sizes that fill their MFMA tiles take the block images as they are (16-byte aligned images); the
-  // others are staged through registers, which pads them.  The tuning switch paged_prefill_dma = 0 forces the staged form.
-  const bool dma = p.d == hdp && p.vc_block % 8 == 0 && p.vc_head % 8 == 0 && tuning().paged_prefill_dma != 0;
-#define HA_W8P(H)                                              \
-  if (dma) launch_prefill_w8<T, H, W8_PAGED_DMA>(p, stream);   \
+  // The block images go into LDS as they are (16-byte aligned images); head sizes that fill their MFMA tiles
+  // take the plain form, those from 40 up that do not take the form that clears what an image leaves
+  // untouched, the rest is staged through registers, which pads it.  The tuning switch paged_prefill_dma = 0
+  // forces the staged form.
+  const bool dma = p.vc_block % 8 == 0 && p.vc_head % 8 == 0 && tuning().paged_prefill_dma != 0;
+#define HA_W8P(H)                                                                  \
+  if (dma && p.d == H) launch_prefill_w8<T, H, W8_PAGED_DMA>(p, stream);           \
+  else if (dma && H >= 64) launch_prefill_w8<T, (H >= 64 ? H : 64), W8_PAGED_DMA_PART>(p, stream); \
   else launch_prefill_w8<T, H, W8_PAGED>(p, stream)
   switch (hdp) {
     case 32: HA_W8P(32); break;

@@ -19,9 +19,10 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(autouse=True, params=["auto", "staged"])
 def tile_route(request, tuning):
-    """Head sizes that fill their MFMA tiles (32, 64, 96, 128) have their tiles copied from the cache into
-    LDS as block images; the others -- and every size when the tuning switch paged_prefill_dma is 0 -- are staged
-    through registers.  Every test runs both ways."""
+    """Head sizes from 40 up (and 32) have their tiles copied from the cache into LDS as block images -- those
+    that do not fill their MFMA tiles (40, 72, 80, 104, ...) with the rest of each image's place cleared; the
+    smaller ones -- and every size when the tuning switch paged_prefill_dma is 0 -- are staged through
+    registers.  Every test runs both ways."""
     tuning("paged_prefill_dma", -1 if request.param == "auto" else 0)
     return request.param
 
@@ -75,7 +76,7 @@ SEQS = [(0, 5), (0, 64), (100, 33), (1000, 256), (17, 1), (0, 300), (63, 65), (2
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("heads", [(32, 8, 128), (32, 32, 80), (8, 2, 64), (4, 4, 32), (6, 1, 96), (8, 2, 112), (4, 4, 120),
-                                   (4, 2, 8)])
+                                   (4, 2, 8), (4, 2, 40), (4, 4, 72), (2, 1, 104)])
 def test_matches_oracle(device, dtype, heads):
     Hq, Hkv, d = heads
     c = paged_case(31, SEQS, Hq, Hkv, d, dtype, 420)
