@@ -165,7 +165,7 @@ __global__ __launch_bounds__(kThreads) void bias_sample_kernel(SampleParams p) {
     }
   };
 
-  if (greedy) {
+  auto arg_max = [&]() {
     float best = -INFINITY;
     int best_i = 0x7fffffff;
     for (int g = tid; g < groups; g += kThreads) {
@@ -200,6 +200,9 @@ __global__ __launch_bounds__(kThreads) void bias_sample_kernel(SampleParams p) {
         }
       p.out_tokens[seq] = best_i == 0x7fffffff ? 0 : best_i;  // nothing allowed: torch's argmax of equal -inf is 0
     }
+  };
+  if (greedy) {
+    arg_max();
     return;
   }
 
@@ -221,8 +224,16 @@ __global__ __launch_bounds__(kThreads) void bias_sample_kernel(SampleParams p) {
     if (tid == 0) p.out_tokens[seq] = 0;
     return;
   }
-  // A token's probability mass, exp(x - m) in units of 2^-40; below that it counts as nothing.
-  auto mass = [&](float x) -> u64 { return (u64)(__builtin_amdgcn_exp2f((x - m) * kLog2e) * kMassUnit); };
+  if (m == INFINITY) {  // an infinite logit: the softmax is not a distribution (the reference fails); its first holder
+    __syncthreads();
+    arg_max();
+    return;
+  }
+  // A token's probability mass, exp(x - m) in units of 2^-40; below that it counts as nothing.  A token that is
+  // not allowed (-inf, or not a number after the division) has none, whatever the temperature.
+  auto mass = [&](float x) -> u64 {
+    return x > -INFINITY ? (u64)(__builtin_amdgcn_exp2f((x - m) * kLog2e) * kMassUnit) : 0ull;
+  };
 
   u64 z = 0;
   for (int g = tid; g < groups; g += kThreads) {
@@ -310,7 +321,8 @@ __global__ __launch_bounds__(kThreads) void bias_sample_kernel(SampleParams p) {
   }
 
   // The draw, in id order: thread t owns the contiguous token groups [t C, (t + 1) C).
-  const u64 c = (u64)((double)p.uniforms[seq] * (double)total);
+  const float u = fminf(fmaxf(p.uniforms[seq], 0.f), 1.f);  // outside [0, 1): the first or the last kept token
+  const u64 c = (u64)((double)u * (double)total);
   const int C = (groups + kThreads - 1) / kThreads;
   const int g_begin = min(tid * C, groups), g_end = min(g_begin + C, groups);
   u64 my_gt = 0;

@@ -332,7 +332,11 @@ char *hipattn_bias_argmax(const hipattn_tensor *logits,
  * returned is the first whose cumulative weight in id order exceeds
  * uniforms[s] * (sum of weights), which is what rand's WeightedIndex returns
  * for that draw.  uniforms[s] in [0, 1) comes from the caller, who keeps the
- * random generators (one per sequence in the reference).  out_tokens int32 [S]. */
+ * random generators (one per sequence in the reference); values outside are
+ * clamped.  A token with bias -inf is never drawn, whatever the temperature.
+ * A row that holds +inf (where the reference's softmax has no answer) yields
+ * the first such token, a row with nothing allowed token 0.
+ * out_tokens int32 [S]. */
 char *hipattn_bias_sample(const hipattn_tensor *logits,
                           const hipattn_tensor *bias,
                           const hipattn_tensor *mask,

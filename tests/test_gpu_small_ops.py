@@ -286,6 +286,33 @@ def test_bias_sample_equal_values_and_distribution(device):
             assert (cum[t - 1] if t else 0.0) - 1e-4 <= float(u[i]) <= cum[t] + 1e-4, (top_p, i, t, int(want[i]))
 
 
+def test_bias_sample_corner_rows(device):
+    """Rows outside what the reference defines still give a defined, allowed token: an infinite logit (its first
+    holder), uniform numbers outside [0, 1) (the first / the last token with weight), an infinite temperature
+    (uniform over the allowed tokens only), nothing allowed (token 0)."""
+    V = 4096
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn((6, V), generator=g).to(torch.bfloat16)
+    allowed = torch.rand((6, V), generator=g) < 0.1
+    allowed[:, 0] = False
+    logits[0, 777] = float("inf")
+    logits[0, 900] = float("inf")
+    allowed[0, 777] = allowed[0, 900] = True
+    allowed[5, :] = False
+    packed = torch.from_numpy(np.stack([aici.pack_allowed(a) for a in allowed.numpy()]))
+    f = lambda *v: torch.tensor(v, dtype=torch.float32, device=device)
+    temperature = f(1.0, 1.0, 1.0, float("inf"), 1e30, 1.0)
+    top_p = f(0.9, 1.0, 1.0, 1.0, 0.5, 0.9)
+    u = f(0.3, -0.5, 7.0, 0.5, 0.999, 0.5)
+    got = K.bias_sample(logits.to(device), temperature, top_p, u, mask=packed.to(device)).tolist()
+    ids = [torch.nonzero(a).flatten().tolist() for a in allowed]
+    assert got[0] == 777
+    assert got[1] == ids[1][0] and got[2] == ids[2][-1]
+    assert got[3] == ids[3][len(ids[3]) // 2]              # equal weights: the middle one at u = 0.5
+    assert got[4] in ids[4]
+    assert got[5] == 0
+
+
 def test_bias_sample_argument_errors(device):
     lg = torch.zeros((2, 64), dtype=torch.float16, device=device)
     f = lambda *v: torch.tensor(v, dtype=torch.float32, device=device)
