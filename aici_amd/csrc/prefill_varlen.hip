@@ -54,11 +54,15 @@
 
 // Phase timeline of one workgroup of the eight-wavefront kernel: built with
 // -DHIPATTN_PHASE_TRACE=<workgroup id>, lane 0 of every wavefront of that
-// workgroup stores the constant-rate 100 MHz counter at the phase boundaries
-// of its first 64 tiles; hipattn_debug_phase_trace copies the table out.  Not
-// compiled into normal builds.
+// workgroup stores a clock at the phase boundaries of its first 64 tiles (the
+// constant-rate 100 MHz counter, or with -DHIPATTN_PHASE_CYCLES the shader
+// clock); hipattn_debug_phase_trace copies the table out.  Not compiled into
+// normal builds.
 #ifdef HIPATTN_PHASE_TRACE
 __device__ long long g_phase_trace[64 * 8 * 8];
+#ifdef HIPATTN_PHASE_CYCLES
+#define wall_clock64 __builtin_readcyclecounter
+#endif
 #define PHASE_STAMP(slot)                                                                                        \
   do {                                                                                                           \
     if (blockIdx.x == HIPATTN_PHASE_TRACE && j < 64 && lane == 0) g_phase_trace[(j * 8 + wave) * 8 + (slot)] = wall_clock64(); \
@@ -692,7 +696,8 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     const unsigned hi = __builtin_amdgcn_readlane((int)(uint32_t)(tbl_off >> 32), idx);
     const char *src = dma_base + (((uint64_t)hi << 32) | lo);
     // the instruction's offset field moves both ends of the copy: the address in memory and the one in LDS
-    const unsigned dst = lds0 + (unsigned)(((tile % NST) * STAGE_ELEMS + dma_v * K_ELEMS + dma_r * BLK_ELEMS) * (int)sizeof(T));
+    const unsigned dst = (unsigned)__builtin_amdgcn_readfirstlane(
+        (int)(lds0 + (unsigned)(((tile % NST) * STAGE_ELEMS + dma_v * K_ELEMS + dma_r * BLK_ELEMS) * (int)sizeof(T))));
 #define HA_DMA_PIECE(OFF)                                                                          \
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:" #OFF \
                :                                                                                   \
@@ -931,7 +936,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   // Tiles entirely past the diagonal of every row of this wavefront are skipped.
   auto skip_tile = [&](int j) { return (wave_row0 >= Lq) || (p.causal && j * BN > wave_last_row + off); };
 
-  // ---- the pipelined tile loop -------------------------------------------------
+  // ---- the pipelined tile loop (staged tiles; block images run the alternating blocks further down) ----
   // Iteration j of a wavefront: the matrix pipe computes S(j+1) = K(j+1).Q^T while
   // the vector ALU turns S(j) into probabilities -- one MFMA is issued, then the
   // few softmax instructions that fit in its shadow, and so on -- then P(j).V(j)
@@ -1015,18 +1020,30 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     l_run += psum;
   };
 
-  // P(j).V(j) with the staging for later tiles in its shadow.
   constexpr int PV_STEPS = NDT * 4;
-  auto pv_stage = [&](bool live, int j, vec8(&pk)[2][2]) {
-    const T *vs_base = smem + (j % NST) * STAGE_ELEMS + K_ELEMS;
-    // Step n = (contraction step n / NDT, output tile n % NDT): consecutive MFMAs go to different
-    // accumulators, so none waits for the result of the one before it.
-    auto rd = [&](int n) -> vec8 {
-      const int dt = n % NDT, ks = n / NDT, kt = ks / 2, half = ks % 2;
-      if constexpr (DMA) return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + ks * (HDP * 16) + dt * 512);
-      return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + dt * 32 * TL::VTSTR + kt * 32 + half * 16);
-    };
-    if (live) {
+  f32x16_t s_a[2], s_b[2];
+  if constexpr (DMA) {
+    // ---- block images: the two wavefronts of a SIMD alternate between the matrix pipe and the vector ALU ----
+    // A wavefront that issues MFMAs and vector instructions in turn has its vector instructions held up
+    // behind every MFMA that waits for the pipe, and its SIMD mate, doing the same, does not fill the gaps
+    // (measured with stamps: the older wavefront of a SIMD needed 3100 cycles per tile and then waited 1600
+    // at the barrier for the younger one).  Here a wavefront runs pure blocks instead -- M(t): the 32 MFMAs of
+    // P(t-1).V(t-1) and S(t); V(t): the softmax of S(t), then the wait for this wavefront's image of a later
+    // tile and the copy of the next one -- and wavefronts 0-3 are half a period ahead of 4-7, so that on
+    // every SIMD one wavefront is in an M block while the other is in a V block.  A barrier ends every half
+    // period h: wavefronts 0-3 run M(t) at h = 2t and V(t) at h = 2t + 1, wavefronts 4-7 M(t) at 2t + 1 and
+    // V(t) at 2t + 2.  Tile T is last read at h = 2T + 3, so its stage (one of four) may be written from
+    // h = 2T + 4 on, i.e. tile T' = T + 4 from h = 2T' - 4, and must be complete before h = 2T': wavefronts
+    // 0-3 copy tile t + 2 in V(t) and wait for it in V(t + 1), wavefronts 4-7 tile t + 3 in V(t).
+    // Measured on 8 x 4096 tokens from the paged cache: 1.118 -> 1.058 ms.
+    vec8 pk[2][2];
+    auto pv_images = [&](int j) {
+      const T *vs_base = smem + (j % NST) * STAGE_ELEMS + K_ELEMS;
+      // Step n = (contraction step n / NDT, output tile n % NDT): consecutive MFMAs go to different
+      // accumulators, so none waits for the result of the one before it.
+      auto rd = [&](int n) -> vec8 {
+        return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + (n / NDT) * (HDP * 16) + (n % NDT) * 512);
+      };
       vec8 va[4];
 #pragma unroll
       for (int n = 0; n < 3 && n < PV_STEPS; n++) va[n] = rd(n);
@@ -1036,63 +1053,112 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         __builtin_amdgcn_sched_barrier(0);
         acc[n % NDT] = Mfma32<T>::run(va[n % 4], pk[(n / NDT) / 2][(n / NDT) % 2], acc[n % NDT]);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (DMA) {
-          // one piece every few MFMAs: issued back to back they queue up in front of the memory pipeline
-          if (n % (PV_STEPS / NDMA) == 1 && j + 3 < n_tiles) {
-            dma_piece(j + 3, n / (PV_STEPS / NDMA));
+      }
+    };
+    auto m_block = [&](int t) {
+      if (t >= 1 && !skip_tile(t - 1)) pv_images(t - 1);
+      if (t < n_tiles && !skip_tile(t)) phase_qk(t % NST, s_a);
+    };
+    // `ahead`: this wavefront's image of tile t + ahead was copied a period ago and is waited for here; the
+    // one of tile t + ahead + 1 follows.  `copy` is false where the prologue has done both already.
+    auto v_block = [&](int t, int ahead, bool copy) {
+      if (!skip_tile(t)) qk_softmax(std::false_type{}, t, s_a, s_b, pk);
+      if (copy) {
+        if (t + ahead < n_tiles) dma_wait(t + ahead, false);
+        if (t + ahead + 1 < n_tiles) dma_tile(t + ahead + 1);
+      }
+    };
+    // The prologue has copied tiles 0, 1 and 2.  Tile 0 has landed; wait for this wavefront's image of tile 1.
+    const bool second_group = wave_u >= 4;
+    if (!second_group) m_block(0);  // h = 0
+    if (n_tiles > 1) dma_wait(1, n_tiles > 2);
+    lds_barrier();
+    if (!second_group) {
+      for (int j = 0; j < n_tiles; j++) {
+        PHASE_STAMP(0);
+        v_block(j, 1, j >= 1);
+        PHASE_STAMP(1);
+        lds_barrier();
+        PHASE_STAMP(2);
+        m_block(j + 1);
+        PHASE_STAMP(3);
+        lds_barrier();
+      }
+      lds_barrier();  // the other group's last product still reads its tile
+    } else {
+      for (int j = 0; j < n_tiles; j++) {
+        PHASE_STAMP(0);
+        m_block(j);
+        PHASE_STAMP(1);
+        lds_barrier();
+        PHASE_STAMP(2);
+        v_block(j, 2, true);
+        PHASE_STAMP(3);
+        lds_barrier();
+      }
+      m_block(n_tiles);
+      lds_barrier();
+    }
+  } else {
+    // ---- staged tiles: one software-pipelined loop per wavefront ----
+    // P(j).V(j) with the staging for later tiles in its shadow.
+    auto pv_stage = [&](bool live, int j, vec8(&pk)[2][2]) {
+      const T *vs_base = smem + (j % NST) * STAGE_ELEMS + K_ELEMS;
+      // Step n = (contraction step n / NDT, output tile n % NDT): consecutive MFMAs go to different
+      // accumulators, so none waits for the result of the one before it.
+      auto rd = [&](int n) -> vec8 {
+        const int dt = n % NDT, ks = n / NDT, kt = ks / 2, half = ks % 2;
+        return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + dt * 32 * TL::VTSTR + kt * 32 + half * 16);
+      };
+      if (live) {
+        vec8 va[4];
+#pragma unroll
+        for (int n = 0; n < 3 && n < PV_STEPS; n++) va[n] = rd(n);
+#pragma unroll
+        for (int n = 0; n < PV_STEPS; n++) {
+          if (n + 3 < PV_STEPS) va[(n + 3) % 4] = rd(n + 3);
+          __builtin_amdgcn_sched_barrier(0);
+          acc[n % NDT] = Mfma32<T>::run(va[n % 4], pk[(n / NDT) / 2][(n / NDT) % 2], acc[n % NDT]);
+          __builtin_amdgcn_sched_barrier(0);
+          if (n == 1) {
+            if (j + 2 < n_tiles) store_tile((j + 2) % 3);
+            if (j + 3 < n_tiles) load_tile(j + 3);
             __builtin_amdgcn_sched_barrier(0);
           }
         }
-        if (n == 1) {
-          if constexpr (!DMA) {
-            if (j + 2 < n_tiles) store_tile((j + 2) % 3);
-            if (j + 3 < n_tiles) load_tile(j + 3);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
+      } else {
+        if (j + 2 < n_tiles) store_tile((j + 2) % 3);
+        if (j + 3 < n_tiles) load_tile(j + 3);
       }
-    } else if constexpr (DMA) {
-      if (j + 3 < n_tiles) dma_tile(j + 3);
-    } else {
-      if (j + 2 < n_tiles) store_tile((j + 2) % 3);
-      if (j + 3 < n_tiles) load_tile(j + 3);
-    }
-  };
+    };
 
-  f32x16_t s_a[2], s_b[2];
-  // S(0) has nothing to hide behind; tile 1 is staged while it runs.
-  if (n_tiles > 0 && !skip_tile(0)) phase_qk(0, s_a);
-  if constexpr (DMA) {
-    if (n_tiles > 1) dma_wait(1, n_tiles > 2);
-  } else {
+    // S(0) has nothing to hide behind; tile 1 is staged while it runs.
+    if (n_tiles > 0 && !skip_tile(0)) phase_qk(0, s_a);
     if (n_tiles > 1) store_tile(1);
     if (n_tiles > 2) load_tile(2);
-  }
-  lds_barrier();
-
-  auto iteration = [&](int j, f32x16_t(&s)[2], f32x16_t(&sn)[2]) {
-    const bool live = !skip_tile(j);
-    const bool live_next = j + 1 < n_tiles && !skip_tile(j + 1);
-    vec8 pk[2][2];
-    PHASE_STAMP(0);
-    if (live) {
-      if (live_next)
-        qk_softmax(std::true_type{}, j, s, sn, pk);
-      else
-        qk_softmax(std::false_type{}, j, s, sn, pk);
-    }
-    PHASE_STAMP(1);
-    pv_stage(live, j, pk);
-    PHASE_STAMP(2);
-    if constexpr (DMA) {
-      if (j + 2 < n_tiles) dma_wait(j + 2, j + 3 < n_tiles);
-    }
     lds_barrier();
-    PHASE_STAMP(3);
-  };
-  for (int j = 0; j < n_tiles; j += 2) {
-    iteration(j, s_a, s_b);
-    if (j + 1 < n_tiles) iteration(j + 1, s_b, s_a);
+
+    auto iteration = [&](int j, f32x16_t(&s)[2], f32x16_t(&sn)[2]) {
+      const bool live = !skip_tile(j);
+      const bool live_next = j + 1 < n_tiles && !skip_tile(j + 1);
+      vec8 pk[2][2];
+      PHASE_STAMP(0);
+      if (live) {
+        if (live_next)
+          qk_softmax(std::true_type{}, j, s, sn, pk);
+        else
+          qk_softmax(std::false_type{}, j, s, sn, pk);
+      }
+      PHASE_STAMP(1);
+      pv_stage(live, j, pk);
+      PHASE_STAMP(2);
+      lds_barrier();
+      PHASE_STAMP(3);
+    };
+    for (int j = 0; j < n_tiles; j += 2) {
+      iteration(j, s_a, s_b);
+      if (j + 1 < n_tiles) iteration(j + 1, s_b, s_a);
+    }
   }
 
   // ---- epilogue ---------------------------------------------------------------
