@@ -469,15 +469,21 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   typedef typename Vec8<T>::type vec8;
   typedef TileW8<HDP> TL;
   constexpr bool PAGED = MODE != W8_ROWS;
+  constexpr bool ROWS = MODE == W8_ROWS;
   constexpr bool DMA = MODE == W8_PAGED_DMA || MODE == W8_PAGED_DMA_PART;
+  // W8_ROWS: K tiles are copied global -> LDS into the layout of the cache's block images (16-byte runs of a
+  // row of k are the images' units, so a lane address per run is all it takes), V tiles are transposed
+  // through registers.  Both forms run the alternating MFMA / softmax blocks.
+  constexpr bool KIMG = DMA || ROWS;      // K tiles lie in LDS as block images
+  constexpr bool PINGPONG = DMA || ROWS;
   // W8_PAGED_DMA_PART: head sizes below HDP (Phi-2's 80 in the 96-wide instance).  An image then fills only the
   // first d / HDP of its place in LDS; the rest is cleared once, so the contraction steps and output rows past d
   // work on zeros.
   constexpr bool DMA_PART = MODE == W8_PAGED_DMA_PART;
   // W8_PAGED_DMA keeps a tile as the four block images of the cache, unpadded, in four stages.
-  constexpr int NST = DMA ? 4 : 3;
-  constexpr int STAGE_ELEMS = DMA ? 2 * BN * HDP : TL::STAGE_ELEMS;
-  constexpr int K_ELEMS = DMA ? BN * HDP : TL::K_ELEMS;
+  constexpr int NST = PINGPONG ? 4 : 3;
+  constexpr int K_ELEMS = KIMG ? BN * HDP : TL::K_ELEMS;
+  constexpr int STAGE_ELEMS = DMA ? 2 * BN * HDP : K_ELEMS + TL::V_ELEMS;
   constexpr int KSTEPS = HDP / 16;
   constexpr int NDT = HDP / 32;
   constexpr int CPR = HDP / 8;                // 16-byte chunks per K row
@@ -603,12 +609,6 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   // Per-thread byte offsets inside a tile, relative to its first key, in 32
   // bits (the launcher checks that 64 rows fit): a full tile's loads are then
   // a uniform base plus a 32-bit lane offset.
-  uint32_t k_boff[NLOADK];
-#pragma unroll
-  for (int i = 0; i < NLOADK; i++) {
-    const int idx = min(tid + 512 * i, K_CHUNKS - 1);
-    k_boff[i] = (uint32_t)(((int64_t)(idx / CPR) * p.k_row + min(idx % CPR, d_chunks - 1) * 8) * (int64_t)sizeof(T));
-  }
   const uint32_t v_boff = (uint32_t)(((int64_t)(v_kg4 * 4) * p.v_row + min(v_dg, p.d / 4 - 1) * 4) * (int64_t)sizeof(T));
   // PAGED: blocks of the cache instead of rows of k / v.  A tile is 4 blocks; threads follow the cache's
   // own order so that consecutive lanes read consecutive 16-byte runs: K unit u = (block, chunk c8,
@@ -767,23 +767,15 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       }
     }
   };
-  auto load_tile_rows = [&](int tile) {
+  // W8_ROWS, V: thread t's block of 4 keys x 4 head elements of the tile.
+  auto load_v_rows = [&](int tile) {
     const int k0 = tile * BN;
     if (k0 + BN <= Lk) {
-      const char *kt = reinterpret_cast<const char *>(kp + (int64_t)k0 * p.k_row);
       const char *vt = reinterpret_cast<const char *>(vp + (int64_t)k0 * p.v_row);
-#pragma unroll
-      for (int i = 0; i < NLOADK; i++) kst[i] = *reinterpret_cast<const u32x4_t *>(kt + k_boff[i]);
 #pragma unroll
       for (int kk = 0; kk < 4; kk++)
         vst[0][kk] = *reinterpret_cast<const u32x2_t *>(vt + (int64_t)kk * p.v_row * (int64_t)sizeof(T) + v_boff);
     } else {  // the last, partial tile: clamp every key to the last real one
-#pragma unroll
-      for (int i = 0; i < NLOADK; i++) {
-        const int idx = min(tid + 512 * i, K_CHUNKS - 1);
-        const int key = min(k0 + idx / CPR, Lk - 1);
-        kst[i] = *reinterpret_cast<const u32x4_t *>(kp + (int64_t)key * p.k_row + min(idx % CPR, d_chunks - 1) * 8);
-      }
 #pragma unroll
       for (int kk = 0; kk < 4; kk++) {
         const int key = min(k0 + v_kg4 * 4 + kk, Lk - 1);
@@ -791,12 +783,43 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       }
     }
   };
-  auto load_tile = [&](int tile) {
-    if constexpr (PAGED)
-      load_tile_paged(tile);
-    else
-      load_tile_rows(tile);
+  // W8_ROWS, K: the tile goes global -> LDS in 1 KiB pieces, 4 x HDP / 32 of them, dealt round the
+  // wavefronts.  Piece q is runs [4 pi .. 4 pi + 4) x 16 tokens of block r = q / (HDP / 32), pi = q %
+  // (HDP / 32), of the image layout [run][token][8 elements]: lane l fetches run 4 pi + l / 16 of token
+  // l % 16.  On a full tile the lane's offset is the same for every piece (the piece's own part is added to
+  // the scalar base); only the last piece of a block clamps runs past d, and the last tile keys past Lk.
+  constexpr int KPB = HDP / 32;   // pieces per block
+  constexpr int KNP = 4 * KPB;    // pieces per tile
+  const int kd_tok = lane & 15, kd_run = lane >> 4;
+  const uint32_t kd_off = (uint32_t)(((int64_t)kd_tok * p.k_row + kd_run * 8) * (int64_t)sizeof(T));
+  const uint32_t kd_off_last =
+      (uint32_t)(((int64_t)kd_tok * p.k_row + (min(4 * (KPB - 1) + kd_run, d_chunks - 1) - 4 * (KPB - 1)) * 8) * (int64_t)sizeof(T));
+  auto k_rows_dma = [&](int tile) {
+    const int k0 = tile * BN;
+    const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem_raw;
+#pragma unroll
+    for (int i = 0; i < (KNP + 7) / 8; i++) {
+      const int q = wave_u + 8 * i;
+      if (KNP % 8 == 0 || q < KNP) {
+        const int r = q / KPB, pi = q % KPB;
+        uint32_t off = pi == KPB - 1 ? kd_off_last : kd_off;
+        int64_t first = (int64_t)(k0 + 16 * r) * p.k_row + 32 * pi;  // elements from kp; uniform
+        if (k0 + BN > Lk) {
+          const int key = min(k0 + 16 * r + kd_tok, Lk - 1);
+          off = (uint32_t)(((int64_t)(key - k0) * p.k_row + (min(4 * pi + kd_run, d_chunks - 1) - 4 * pi) * 8) * (int64_t)sizeof(T));
+          first = (int64_t)k0 * p.k_row + 32 * pi;
+        }
+        const T *src = kp + first;
+        const unsigned dst = (unsigned)__builtin_amdgcn_readfirstlane(
+            (int)(lds_base + (unsigned)(((tile % NST) * STAGE_ELEMS + r * (HDP * 16)) * (int)sizeof(T)) + pi * 1024));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(dst), "v"(off), "s"(src)
+                     : "memory", "m0");
+      }
+    }
   };
+  auto load_tile = [&](int tile) { load_tile_paged(tile); };
   auto store_tile_paged = [&](int stage) {
     T *ks = smem + stage * STAGE_ELEMS;
     T *vs = ks + K_ELEMS;
@@ -833,43 +856,25 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       }
     }
   };
-  auto store_tile_rows = [&](int stage) {
-    T *ks = smem + stage * STAGE_ELEMS;
-    T *vs = ks + K_ELEMS;
+  // W8_ROWS, V: the thread's block transposed in registers and written into V^T, keys in their own order (the
+  // order in which the image layout of K hands the scores to the second product).
+  auto store_v_rows = [&](int stage) {
+    T *vs = smem + stage * STAGE_ELEMS + K_ELEMS;
+    if (V_ITEMS % 512 == 0 || v_dg < HDP / 4) {
+      // 4x4 transpose of 16-bit values: out[dd] = {k0.d, k1.d, k2.d, k3.d}
+      const unsigned a0 = vst[0][0][0], a1 = vst[0][0][1], b0 = vst[0][1][0], b1 = vst[0][1][1];
+      const unsigned c0 = vst[0][2][0], c1 = vst[0][2][1], e0 = vst[0][3][0], e1 = vst[0][3][1];
+      u32x2_t o[4];
+      o[0] = u32x2_t{__builtin_amdgcn_perm(b0, a0, 0x05040100u), __builtin_amdgcn_perm(e0, c0, 0x05040100u)};
+      o[1] = u32x2_t{__builtin_amdgcn_perm(b0, a0, 0x07060302u), __builtin_amdgcn_perm(e0, c0, 0x07060302u)};
+      o[2] = u32x2_t{__builtin_amdgcn_perm(b1, a1, 0x05040100u), __builtin_amdgcn_perm(e1, c1, 0x05040100u)};
+      o[3] = u32x2_t{__builtin_amdgcn_perm(b1, a1, 0x07060302u), __builtin_amdgcn_perm(e1, c1, 0x07060302u)};
 #pragma unroll
-    for (int i = 0; i < NLOADK; i++) {
-      const int idx = tid + 512 * i;
-      if (K_CHUNKS % 512 == 0 || idx < K_CHUNKS) {
-        const int row = idx / CPR, ch = idx % CPR;
-        *reinterpret_cast<u32x4_t *>(ks + row * TL::KSTR + ch * 8) = kst[i];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < NLOADV; i++) {
-      if (V_ITEMS % 512 == 0 || v_dg < HDP / 4) {
-        // 4x4 transpose of 16-bit values: out[dd] = {k0.d, k1.d, k2.d, k3.d}
-        const unsigned a0 = vst[i][0][0], a1 = vst[i][0][1], b0 = vst[i][1][0], b1 = vst[i][1][1];
-        const unsigned c0 = vst[i][2][0], c1 = vst[i][2][1], e0 = vst[i][3][0], e1 = vst[i][3][1];
-        u32x2_t o[4];
-        o[0] = u32x2_t{__builtin_amdgcn_perm(b0, a0, 0x05040100u), __builtin_amdgcn_perm(e0, c0, 0x05040100u)};
-        o[1] = u32x2_t{__builtin_amdgcn_perm(b0, a0, 0x07060302u), __builtin_amdgcn_perm(e0, c0, 0x07060302u)};
-        o[2] = u32x2_t{__builtin_amdgcn_perm(b1, a1, 0x05040100u), __builtin_amdgcn_perm(e1, c1, 0x05040100u)};
-        o[3] = u32x2_t{__builtin_amdgcn_perm(b1, a1, 0x07060302u), __builtin_amdgcn_perm(e1, c1, 0x07060302u)};
-        // Key offset within its group of 16: bits [a(8) g(4) b(2,1)] -> position [g(8) a(4) b].
-        const int o16 = (v_kg4 & 3) * 4;
-        const int pos = (v_kg4 >> 2) * 16 + ((o16 & 4) << 1) + ((o16 & 8) >> 1);
-#pragma unroll
-        for (int dd = 0; dd < 4; dd++)
-          *reinterpret_cast<u32x2_t *>(vs + (v_dg * 4 + dd) * TL::VTSTR + pos) = o[dd];
-      }
+      for (int dd = 0; dd < 4; dd++)
+        *reinterpret_cast<u32x2_t *>(vs + (v_dg * 4 + dd) * TL::VTSTR + v_kg4 * 4) = o[dd];
     }
   };
-  auto store_tile = [&](int stage) {
-    if constexpr (PAGED)
-      store_tile_paged(stage);
-    else
-      store_tile_rows(stage);
-  };
+  auto store_tile = [&](int stage) { store_tile_paged(stage); };
 
   if (PAGED && n_tiles > 0) tbl_cur = load_ids(0);
   if constexpr (DMA) {
@@ -884,6 +889,22 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     if (n_tiles > 1) dma_tile(1);
     if (n_tiles > 2) dma_tile(2);
     clear_image_tails(1, NST - 1);  // seen by all after the barrier in front of the loop; stage 1 is first read there
+  } else if constexpr (ROWS) {
+    // Tile 0 arrives in stage 0 while Q is turned through stages 1..3; then K of tiles 1 and 2 is copied,
+    // V of tile 1 goes through the registers into its stage and V of tile 2 into the registers.
+    if (n_tiles > 0) {
+      load_v_rows(0);
+      k_rows_dma(0);
+    }
+    load_q();
+    if (n_tiles > 0) store_v_rows(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (n_tiles > 1) {
+      load_v_rows(1);
+      k_rows_dma(1);
+    }
+    if (n_tiles > 2) k_rows_dma(2);
   } else {
     if (n_tiles > 0) load_tile(0);
     load_q();
@@ -900,11 +921,11 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   // a V row lies in the cache.  Sixteen consecutive lanes then read one whole 256-byte run [chunk][16
   // tokens] of K, and the 32 lanes of a half-wavefront 512 consecutive bytes of V (the DMA places the two
   // 8-token halves of 32 rows one after the other): no padding is needed.
-  const int k_lane_off = DMA ? (c >> 4) * (HDP * 16) + g * 128 + (((c >> 2) & 1) * 8 + ((c >> 3) & 1) * 4 + (c & 3)) * 8
-                             : c * TL::KSTR + g * 8;
+  const int k_lane_off = KIMG ? (c >> 4) * (HDP * 16) + g * 128 + (((c >> 2) & 1) * 8 + ((c >> 3) & 1) * 4 + (c & 3)) * 8
+                              : c * TL::KSTR + g * 8;
   const int v_lane_off = DMA ? g * 256 + c * 8 : c * TL::VTSTR + g * 8;
-  constexpr int K_HALF = DMA ? 2 * HDP * 16 : 32 * TL::KSTR;  // elements between the two 32-key halves of a K tile
-  constexpr int K_STEP = DMA ? 256 : 16;                      // ... between contraction steps (16 head elements)
+  constexpr int K_HALF = KIMG ? 2 * HDP * 16 : 32 * TL::KSTR;  // elements between the two 32-key halves of a K tile
+  constexpr int K_STEP = KIMG ? 256 : 16;                      // ... between contraction steps (16 head elements)
   const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // S^T = K . Q^T of one tile on its own (used for tile 0): both 32-key halves,
@@ -979,8 +1000,8 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       for (int kt = 0; kt < 2; kt++)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-          const int key = DMA ? k0 + kt * 32 + ((i >> 3) & 1) * 16 + g * 8 + ((i >> 2) & 1) * 4 + (i & 3)
-                              : k0 + kt * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
+          const int key = KIMG ? k0 + kt * 32 + ((i >> 3) & 1) * 16 + g * 8 + ((i >> 2) & 1) * 4 + (i & 3)
+                               : k0 + kt * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
           if (key > limit) s[kt][i] = -INFINITY;
         }
     }
@@ -1022,8 +1043,8 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
 
   constexpr int PV_STEPS = NDT * 4;
   f32x16_t s_a[2], s_b[2];
-  if constexpr (DMA) {
-    // ---- block images: the two wavefronts of a SIMD alternate between the matrix pipe and the vector ALU ----
+  if constexpr (PINGPONG) {
+    // ---- block images and rows: the two wavefronts of a SIMD alternate between the matrix pipe and the vector ALU ----
     // A wavefront that issues MFMAs and vector instructions in turn has its vector instructions held up
     // behind every MFMA that waits for the pipe, and its SIMD mate, doing the same, does not fill the gaps
     // (measured with stamps: the older wavefront of a SIMD needed 3100 cycles per tile and then waited 1600
@@ -1042,7 +1063,8 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       // Step n = (contraction step n / NDT, output tile n % NDT): consecutive MFMAs go to different
       // accumulators, so none waits for the result of the one before it.
       auto rd = [&](int n) -> vec8 {
-        return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + (n / NDT) * (HDP * 16) + (n % NDT) * 512);
+        if constexpr (DMA) return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + (n / NDT) * (HDP * 16) + (n % NDT) * 512);
+        return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + (n % NDT) * 32 * TL::VTSTR + (n / NDT) * 16);
       };
       vec8 va[4];
 #pragma unroll
@@ -1055,23 +1077,47 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         __builtin_amdgcn_sched_barrier(0);
       }
     };
-    auto m_block = [&](int t) {
+    // W8_ROWS: the V rows that this wavefront asked for in its last V block are transposed and stored behind
+    // the MFMAs, where the wavefront would otherwise wait at the barrier (`ahead` as for v_block).
+    auto m_block = [&](int t, int ahead) {
       if (t >= 1 && !skip_tile(t - 1)) pv_images(t - 1);
       if (t < n_tiles && !skip_tile(t)) phase_qk(t % NST, s_a);
+      if constexpr (ROWS) {
+        if ((t >= 1 || ahead == 2) && t + ahead < n_tiles) store_v_rows((t + ahead) % NST);
+      }
     };
     // `ahead`: this wavefront's image of tile t + ahead was copied a period ago and is waited for here; the
     // one of tile t + ahead + 1 follows.  `copy` is false where the prologue has done both already.
     auto v_block = [&](int t, int ahead, bool copy) {
       if (!skip_tile(t)) qk_softmax(std::false_type{}, t, s_a, s_b, pk);
       if (copy) {
-        if (t + ahead < n_tiles) dma_wait(t + ahead, false);
-        if (t + ahead + 1 < n_tiles) dma_tile(t + ahead + 1);
+        if constexpr (DMA) {
+          if (t + ahead < n_tiles) dma_wait(t + ahead, false);
+          if (t + ahead + 1 < n_tiles) dma_tile(t + ahead + 1);
+        } else {
+          // K of tile t + ahead has landed (its V went into LDS behind the last M block); the next tile follows
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          // The loads first: the compiler counts only its own memory operations when it places waits, and a
+          // wait it puts between these loads would otherwise also wait for the copies just issued.
+          if (t + ahead + 1 < n_tiles) {
+            load_v_rows(t + ahead + 1);
+            k_rows_dma(t + ahead + 1);
+          }
+        }
       }
     };
     // The prologue has copied tiles 0, 1 and 2.  Tile 0 has landed; wait for this wavefront's image of tile 1.
     const bool second_group = wave_u >= 4;
-    if (!second_group) m_block(0);  // h = 0
-    if (n_tiles > 1) dma_wait(1, n_tiles > 2);
+    if (!second_group) m_block(0, 1);  // h = 0
+    if constexpr (DMA) {
+      if (n_tiles > 1) dma_wait(1, n_tiles > 2);
+    } else {
+      if (n_tiles > 1) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        store_v_rows(1);
+      }
+      if (n_tiles > 2) load_v_rows(2);
+    }
     lds_barrier();
     if (!second_group) {
       for (int j = 0; j < n_tiles; j++) {
@@ -1080,7 +1126,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         PHASE_STAMP(1);
         lds_barrier();
         PHASE_STAMP(2);
-        m_block(j + 1);
+        m_block(j + 1, 1);
         PHASE_STAMP(3);
         lds_barrier();
       }
@@ -1088,7 +1134,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     } else {
       for (int j = 0; j < n_tiles; j++) {
         PHASE_STAMP(0);
-        m_block(j);
+        m_block(j, 2);
         PHASE_STAMP(1);
         lds_barrier();
         PHASE_STAMP(2);
@@ -1096,7 +1142,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         PHASE_STAMP(3);
         lds_barrier();
       }
-      m_block(n_tiles);
+      m_block(n_tiles, 2);
       lds_barrier();
     }
   } else {
@@ -1234,7 +1280,9 @@ template <typename T, int HDP, int MODE = W8_ROWS>
 void launch_prefill_w8(PrefillParams p, hipStream_t stream) {
   static bool attr_set = false;  // benign race: setting twice is harmless
   auto kernel = prefill_varlen_w8_kernel<T, HDP, MODE>;
-  constexpr size_t lds_bytes = MODE >= W8_PAGED_DMA ? (size_t)4 * 2 * BN * HDP * 2 : TileW8<HDP>::LDS_BYTES;
+  constexpr size_t lds_bytes = MODE >= W8_PAGED_DMA ? (size_t)4 * 2 * BN * HDP * 2
+                               : MODE == W8_ROWS   ? (size_t)4 * (BN * HDP + TileW8<HDP>::V_ELEMS) * 2
+                                                   : TileW8<HDP>::LDS_BYTES;
   if (!attr_set) {
     HA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)lds_bytes));
