@@ -89,14 +89,16 @@ __global__ __launch_bounds__(256) void cache_move_run8_kernel(
     uint16_t *__restrict__ key, uint16_t *__restrict__ value, uint16_t *__restrict__ key_cache,
     uint16_t *__restrict__ value_cache, const Slot *__restrict__ slot_mapping, int64_t num_tokens,
     int64_t key_tok_stride, int64_t key_head_stride, int64_t val_tok_stride,
-    int64_t val_head_stride, CacheGeom g) {
+    int64_t val_head_stride, CacheGeom g, int heads_per_wg) {
   typedef uint16_t E;
   constexpr int X = 8;
   // 16 tokens per workgroup, as two groups of 8: a block filled in order is then
-  // written by one workgroup, whose half-row stores meet in the same L2.
+  // written by one workgroup, whose half-row stores meet in the same L2.  With few tokens the heads are
+  // dealt over blockIdx.y as well, so that the launch still has workgroups for every CU.
   const int64_t wg_t0 = (int64_t)blockIdx.x * 16;
   const int chunks_per_head = g.head_size / X;
-  const int n = g.num_heads * chunks_per_head;
+  const int h_first = blockIdx.y * heads_per_wg;
+  const int n = min(heads_per_wg, g.num_heads - h_first) * chunks_per_head;
   int64_t run_slot[2];
 #pragma unroll
   for (int half = 0; half < 2; half++) {
@@ -115,7 +117,7 @@ __global__ __launch_bounds__(256) void cache_move_run8_kernel(
   for (int idx = threadIdx.x; idx < 2 * n; idx += blockDim.x) {
     const int half = idx / n;
     const int i = idx % n;
-    const int h = i / chunks_per_head;
+    const int h = h_first + i / chunks_per_head;
     const int c = i % chunks_per_head;
     const int64_t t0 = wg_t0 + 8 * half;
     const int64_t slot0 = half == 0 ? run_slot[0] : run_slot[1];
@@ -164,20 +166,51 @@ __global__ __launch_bounds__(256) void cache_move_run8_kernel(
       }
       continue;
     }
-    // per-token path for this group of 8
+    // per-token path for this group of 8: all slots first, then all loads, then all stores, so that the
+    // eight tokens' memory round trips overlap instead of following one another (decode rows come this way)
+    int64_t slots[8];
+#pragma unroll
     for (int t = 0; t < 8; t++) {
       const int64_t token = t0 + t;
-      if (token >= num_tokens) break;
-      const int64_t slot = (int64_t)slot_mapping[token];
-      if (slot < 0) continue;
-      const int64_t blk = slot / g.block_size;
-      if (blk >= g.num_blocks) continue;
-      const int off = (int)(slot % g.block_size);
-      E *kp = key + token * key_tok_stride + h * key_head_stride + c * X;
-      E *vp = value + token * val_tok_stride + h * val_head_stride + c * X;
-      E *kc = key_cache + blk * g.k_block_stride + h * g.k_head_stride + ((int64_t)c * g.block_size + off) * X;
-      E *vc = value_cache + blk * g.v_block_stride + h * g.v_head_stride + (int64_t)c * X * g.block_size + off;
-      move_token_chunk<E, SCATTER>(kp, vp, kc, vc, g.block_size);
+      int64_t slot = token < num_tokens ? (int64_t)slot_mapping[token] : -1;
+      if (slot >= 0 && slot / g.block_size >= g.num_blocks) slot = -1;
+      slots[t] = slot;
+    }
+    uint4 kk[8], vv[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      kk[t] = vv[t] = uint4{0u, 0u, 0u, 0u};
+      if (slots[t] < 0) continue;
+      const int64_t blk = slots[t] / g.block_size;
+      const int off = (int)(slots[t] % g.block_size);
+      if (SCATTER) {
+        kk[t] = *reinterpret_cast<const uint4 *>(key + (t0 + t) * key_tok_stride + h * key_head_stride + c * X);
+        vv[t] = *reinterpret_cast<const uint4 *>(value + (t0 + t) * val_tok_stride + h * val_head_stride + c * X);
+      } else {
+        kk[t] = *reinterpret_cast<const uint4 *>(key_cache + blk * g.k_block_stride + h * g.k_head_stride +
+                                                 ((int64_t)c * g.block_size + off) * X);
+        const E *vc = value_cache + blk * g.v_block_stride + h * g.v_head_stride + (int64_t)c * X * g.block_size + off;
+        E *ve = reinterpret_cast<E *>(&vv[t]);
+#pragma unroll
+        for (int j = 0; j < X; j++) ve[j] = vc[(int64_t)j * g.block_size];
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      if (slots[t] < 0) continue;
+      const int64_t blk = slots[t] / g.block_size;
+      const int off = (int)(slots[t] % g.block_size);
+      if (SCATTER) {
+        *reinterpret_cast<uint4 *>(key_cache + blk * g.k_block_stride + h * g.k_head_stride +
+                                   ((int64_t)c * g.block_size + off) * X) = kk[t];
+        E *vc = value_cache + blk * g.v_block_stride + h * g.v_head_stride + (int64_t)c * X * g.block_size + off;
+        const E *ve = reinterpret_cast<const E *>(&vv[t]);
+#pragma unroll
+        for (int j = 0; j < X; j++) vc[(int64_t)j * g.block_size] = ve[j];
+      } else {
+        *reinterpret_cast<uint4 *>(key + (t0 + t) * key_tok_stride + h * key_head_stride + c * X) = kk[t];
+        *reinterpret_cast<uint4 *>(value + (t0 + t) * val_tok_stride + h * val_head_stride + c * X) = vv[t];
+      }
     }
   }
 }
@@ -543,10 +576,17 @@ void launch_move(const hipattn_tensor *key, const hipattn_tensor *value,
         check_launch(SCATTER ? "reshape_and_cache" : "gather_cached_kv");
         return;
       }
-      int n = g.num_heads * (g.head_size / X);
+      // about two thousand workgroups, if the heads allow: a few hundred of them leave most of the memory
+      // system idle (2168 tokens of 32 heads x 80: 60 us with one workgroup per 16 tokens)
+      const int64_t groups = (T + 15) / 16;
+      int slices = (int)std::min<int64_t>(g.num_heads, (2048 + groups - 1) / groups);
+      const int heads_per_wg = (g.num_heads + slices - 1) / slices;
+      slices = (g.num_heads + heads_per_wg - 1) / heads_per_wg;
+      int n = 2 * heads_per_wg * (g.head_size / X);
       int threads = n < 256 ? ((n + 63) / 64) * 64 : 256;
-      cache_move_run8_kernel<Slot, SCATTER><<<dim3((unsigned)((T + 15) / 16)), threads, 0, stream>>>(
-          kp, vp, kc, vc, sp, T, key->strides[0], key->strides[1], value->strides[0], value->strides[1], g);
+      cache_move_run8_kernel<Slot, SCATTER><<<dim3((unsigned)groups, (unsigned)slices), threads, 0, stream>>>(
+          kp, vp, kc, vc, sp, T, key->strides[0], key->strides[1], value->strides[0], value->strides[1], g,
+          heads_per_wg);
       check_launch(SCATTER ? "reshape_and_cache" : "gather_cached_kv");
       return;
     }
