@@ -152,8 +152,12 @@ def aici_greedy(logits: torch.Tensor, allow_masks: torch.Tensor) -> torch.Tensor
 
 
 def aici_sample(logits: torch.Tensor, allow_masks: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
-                uniforms: torch.Tensor) -> torch.Tensor:
+                uniforms: torch.Tensor = None, generator: torch.Generator = None) -> torch.Tensor:
     """The sampling half with temperature and top-p (tmodel.rs:172-194, 236-268) under the same packed
-    allow-masks: rows with temperature < 1e-5 are greedy, the others are drawn with the caller's uniform
-    numbers (one per row, in [0, 1)).  All rows in one launch, no host round trip.  Returns int32 [S]."""
+    allow-masks: rows with temperature < 1e-5 are greedy, the others are drawn with one uniform number per
+    row in [0, 1) -- the caller's, or drawn here from `generator` (a seeded torch.Generator on the CPU stands
+    in for the reference's per-sequence `StdRng`: the same seed gives the same tokens).  All rows in one
+    launch, no host round trip.  Returns int32 [S]."""
+    if uniforms is None:
+        uniforms = torch.rand((logits.size(0),), generator=generator, dtype=torch.float32).to(logits.device)
     return kernels.bias_sample(logits, temperature, top_p, uniforms, mask=allow_masks)

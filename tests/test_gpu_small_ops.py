@@ -313,6 +313,28 @@ def test_bias_sample_corner_rows(device):
     assert got[5] == 0
 
 
+def test_aici_sample_with_a_seeded_generator(device):
+    """llama.aici_sample draws its uniform numbers from a seeded generator when none are given: the same seed
+    gives the same tokens, those the oracle picks for the same numbers, and only allowed ones."""
+    from aici_amd import llama
+    S, V = 16, 32000
+    g = torch.Generator().manual_seed(21)
+    logits = (torch.randn((S, V), generator=g) * 3).to(torch.bfloat16)
+    allowed = torch.rand((S, V), generator=g) < 0.02
+    packed = torch.from_numpy(np.stack([aici.pack_allowed(a) for a in allowed.numpy()]))
+    temperature = torch.full((S,), 0.7, device=device)
+    top_p = torch.full((S,), 0.95, device=device)
+    draw = lambda seed: llama.aici_sample(logits.to(device), packed.to(device), temperature, top_p,
+                                          generator=torch.Generator().manual_seed(seed)).cpu()
+    a, b, c = draw(5), draw(5), draw(6)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+    assert all(allowed[s, int(a[s])] for s in range(S))
+    u = torch.rand((S,), generator=torch.Generator().manual_seed(5), dtype=torch.float32)
+    bias = torch.where(allowed, 0.0, float("-inf"))
+    differ = _sample_check(logits, bias, temperature.cpu(), top_p.cpu(), u, a)
+    assert differ <= 1
+
+
 def test_bias_sample_argument_errors(device):
     lg = torch.zeros((2, 64), dtype=torch.float16, device=device)
     f = lambda *v: torch.tensor(v, dtype=torch.float32, device=device)
