@@ -481,12 +481,12 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   // work on zeros.
   constexpr bool DMA_PART = MODE == W8_PAGED_DMA_PART;
   // W8_PAGED_DMA keeps a tile as the four block images of the cache, unpadded, in four stages.
-  // Block images: five stages (all of the 160 KB at head size 128) and one barrier per tile; rows: four stages
-  // (a fifth does not fit beside the padded V^T tiles) and a barrier per half period; staged: three.
-  constexpr bool ONE_BARRIER = DMA;
-  constexpr int NST = DMA ? 5 : (PINGPONG ? 4 : 3);
+  // Block images and rows: five stages (all of the 160 KB at head size 128) and one barrier per tile; staged:
+  // three.  For five to fit, the V^T tiles of the rows form are not padded but swizzled: the 16-byte run q of
+  // row r lies at run q ^ ((r >> 1) & 7), which keeps the operand reads free of bank conflicts.
+  constexpr int NST = PINGPONG ? 5 : 3;
   constexpr int K_ELEMS = KIMG ? BN * HDP : TL::K_ELEMS;
-  constexpr int STAGE_ELEMS = DMA ? 2 * BN * HDP : K_ELEMS + TL::V_ELEMS;
+  constexpr int STAGE_ELEMS = PINGPONG ? 2 * BN * HDP : K_ELEMS + TL::V_ELEMS;
   constexpr int KSTEPS = HDP / 16;
   constexpr int NDT = HDP / 32;
   constexpr int CPR = HDP / 8;                // 16-byte chunks per K row
@@ -873,8 +873,10 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       o[2] = u32x2_t{__builtin_amdgcn_perm(b1, a1, 0x05040100u), __builtin_amdgcn_perm(e1, c1, 0x05040100u)};
       o[3] = u32x2_t{__builtin_amdgcn_perm(b1, a1, 0x07060302u), __builtin_amdgcn_perm(e1, c1, 0x07060302u)};
 #pragma unroll
-      for (int dd = 0; dd < 4; dd++)
-        *reinterpret_cast<u32x2_t *>(vs + (v_dg * 4 + dd) * TL::VTSTR + v_kg4 * 4) = o[dd];
+      for (int dd = 0; dd < 4; dd++) {
+        const int r = v_dg * 4 + dd;
+        *reinterpret_cast<u32x2_t *>(vs + r * BN + (((v_kg4 >> 1) ^ ((r >> 1) & 7)) * 8) + (v_kg4 & 1) * 4) = o[dd];
+      }
     }
   };
   auto store_tile = [&](int stage) { store_tile_paged(stage); };
@@ -927,6 +929,11 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   const int k_lane_off = KIMG ? (c >> 4) * (HDP * 16) + g * 128 + (((c >> 2) & 1) * 8 + ((c >> 3) & 1) * 4 + (c & 3)) * 8
                               : c * TL::KSTR + g * 8;
   const int v_lane_off = DMA ? g * 256 + c * 8 : c * TL::VTSTR + g * 8;
+  // W8_ROWS: element offset of run 2 ks + g of this lane's V^T row within a 32-row block, for the four
+  // contraction steps ks of a tile (the swizzle is the same in every block: 32 rows are a multiple of 16)
+  int v_swz_off[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ks++) v_swz_off[ks] = c * BN + (((2 * ks + g) ^ ((c >> 1) & 7)) * 8);
   constexpr int K_HALF = KIMG ? 2 * HDP * 16 : 32 * TL::KSTR;  // elements between the two 32-key halves of a K tile
   constexpr int K_STEP = KIMG ? 256 : 16;                      // ... between contraction steps (16 head elements)
   const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -1055,16 +1062,13 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     // P(t-1).V(t-1) and S(t); V(t): the softmax of S(t), then the wait for this wavefront's image of a later
     // tile and the copy of the next one -- and wavefronts 0-3 are half a period ahead of 4-7, so that on
     // every SIMD one wavefront is in an M block while the other is in a V block.
-    //   Rows: a barrier ends every half period h: wavefronts 0-3 run M(t) at h = 2t and V(t) at h = 2t + 1,
-    // wavefronts 4-7 M(t) at 2t + 1 and V(t) at 2t + 2.  Tile T is last read at h = 2T + 3, so its stage (one of
-    // four) may be written from h = 2T + 4 on, i.e. tile T' = T + 4 from h = 2T' - 4, and must be complete before
-    // h = 2T': wavefronts 0-3 copy tile t + 2 in V(t) and wait for it in V(t + 1), wavefronts 4-7 tile t + 3 in V(t).
-    //   Block images: five stages leave two whole periods between a place becoming free and its tile being
-    // needed, so both groups wait for tile t + 2 and copy tile t + 3 in V(t) and one barrier per period is
-    // enough (a barrier costs the eight wavefronts some 200 cycles): the groups start a period together, one
-    // with its V block, the other with its M block, and swap in the middle.
-    // Measured on 8 x 4096 tokens from the paged cache: 1.118 -> 1.058 ms with two barriers per tile, 1.091 ->
-    // 1.075 ms from two barriers to one.
+    //   Five stages leave two whole periods between a place becoming free and its tile being needed -- tile T
+    // is read in periods T - 1 .. T + 1, its place is that of tile T - 5 -- so both groups wait for tile t + 2
+    // and send tile t + 3 in V(t), and one barrier per period is enough (a barrier costs the eight wavefronts
+    // some 200 cycles): the groups start a period together, wavefronts 0-3 with V(t), wavefronts 4-7 with
+    // M(t), and swap in the middle.
+    // Measured on 8 x 4096 tokens from the paged cache: 1.118 -> 1.058 ms with four stages and a barrier per
+    // half period, 1.091 -> 1.075 ms from there to five stages and one barrier.
     vec8 pk[2][2];
     auto pv_images = [&](int j) {
       const T *vs_base = smem + (j % NST) * STAGE_ELEMS + K_ELEMS;
@@ -1072,7 +1076,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       // accumulators, so none waits for the result of the one before it.
       auto rd = [&](int n) -> vec8 {
         if constexpr (DMA) return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + (n / NDT) * (HDP * 16) + (n % NDT) * 512);
-        return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + (n % NDT) * 32 * TL::VTSTR + (n / NDT) * 16);
+        return *reinterpret_cast<const vec8 *>(vs_base + v_swz_off[n / NDT] + (n % NDT) * 32 * BN);
       };
       vec8 va[4];
 #pragma unroll
@@ -1085,39 +1089,37 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         __builtin_amdgcn_sched_barrier(0);
       }
     };
-    // W8_ROWS: the V rows that this wavefront asked for in its last V block are transposed and stored behind
-    // the MFMAs, where the wavefront would otherwise wait at the barrier (`ahead` as for v_block).
-    auto m_block = [&](int t, int ahead) {
+    // W8_ROWS: the V rows that this wavefront asked for in its last V block (tile t + 2) are transposed and
+    // stored behind the MFMAs, where the wavefront would otherwise wait at the barrier.
+    auto m_block = [&](int t) {
       if (t >= 1 && !skip_tile(t - 1)) pv_images(t - 1);
       if (t < n_tiles && !skip_tile(t)) phase_qk(t % NST, s_a);
       if constexpr (ROWS) {
-        if ((t >= 1 || ahead == 2) && t + ahead < n_tiles) store_v_rows((t + ahead) % NST);
+        if (t + 2 < n_tiles) store_v_rows((t + 2) % NST);
       }
     };
-    // `ahead`: this wavefront's image of tile t + ahead was copied a period ago and is waited for here; the
-    // one of tile t + ahead + 1 follows.  `copy` is false where the prologue has done both already.
-    auto v_block = [&](int t, int ahead, bool copy) {
+    // After the softmax: this wavefront's part of tile t + 2, sent a period ago, is waited for, and its part of
+    // tile t + 3 follows.
+    auto v_block = [&](int t) {
       if (!skip_tile(t)) qk_softmax(std::false_type{}, t, s_a, s_b, pk);
-      if (copy) {
-        if constexpr (DMA) {
-          if (t + ahead < n_tiles) dma_wait(t + ahead, false);
-          if (t + ahead + 1 < n_tiles) dma_tile(t + ahead + 1);
-        } else {
-          // K of tile t + ahead has landed (its V went into LDS behind the last M block); the next tile follows
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-          // The loads first: the compiler counts only its own memory operations when it places waits, and a
-          // wait it puts between these loads would otherwise also wait for the copies just issued.
-          if (t + ahead + 1 < n_tiles) {
-            load_v_rows(t + ahead + 1);
-            k_rows_dma(t + ahead + 1);
-          }
+      if constexpr (DMA) {
+        if (t + 2 < n_tiles) dma_wait(t + 2, false);
+        if (t + 3 < n_tiles) dma_tile(t + 3);
+      } else {
+        // K of tile t + 2 has landed (its V went into LDS behind the last M block)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // The loads first: the compiler counts only its own memory operations when it places waits, and a
+        // wait it puts between these loads would otherwise also wait for the copies just issued.
+        if (t + 3 < n_tiles) {
+          load_v_rows(t + 3);
+          k_rows_dma(t + 3);
         }
       }
     };
-    // The prologue has copied tiles 0, 1 and 2.  Tile 0 has landed; wait for this wavefront's image of tile 1.
+    // The prologue has sent tiles 0, 1 and 2; tiles 0 and 1 have to be complete before the first period.
     const bool second_group = wave_u >= 4;
-    if (!second_group) m_block(0, 1);  // h = 0
     if constexpr (DMA) {
+      if (!second_group) m_block(0);
       if (n_tiles > 1) dma_wait(1, n_tiles > 2);
     } else {
       if (n_tiles > 1) {
@@ -1125,55 +1127,29 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         store_v_rows(1);
       }
       if (n_tiles > 2) load_v_rows(2);
+      if (!second_group) m_block(0);  // its tail stores V of tile 2; the other group's M(0) does so in period 0
     }
     lds_barrier();
-    if constexpr (ONE_BARRIER) {
-      if (!second_group) {
-        for (int j = 0; j < n_tiles; j++) {
-          PHASE_STAMP(0);
-          v_block(j, 2, true);
-          PHASE_STAMP(1);
-          m_block(j + 1, 1);
-          PHASE_STAMP(2);
-          lds_barrier();
-        }
-        lds_barrier();
-      } else {
-        for (int j = 0; j < n_tiles; j++) {
-          PHASE_STAMP(0);
-          m_block(j, 2);
-          PHASE_STAMP(1);
-          v_block(j, 2, true);
-          PHASE_STAMP(2);
-          lds_barrier();
-        }
-        m_block(n_tiles, 2);
-        lds_barrier();
-      }
-    } else if (!second_group) {
+    if (!second_group) {
       for (int j = 0; j < n_tiles; j++) {
         PHASE_STAMP(0);
-        v_block(j, 1, j >= 1);
+        v_block(j);
         PHASE_STAMP(1);
-        lds_barrier();
+        m_block(j + 1);
         PHASE_STAMP(2);
-        m_block(j + 1, 1);
-        PHASE_STAMP(3);
         lds_barrier();
       }
       lds_barrier();  // the other group's last product still reads its tile
     } else {
       for (int j = 0; j < n_tiles; j++) {
         PHASE_STAMP(0);
-        m_block(j, 2);
+        m_block(j);
         PHASE_STAMP(1);
-        lds_barrier();
+        v_block(j);
         PHASE_STAMP(2);
-        v_block(j, 2, true);
-        PHASE_STAMP(3);
         lds_barrier();
       }
-      m_block(n_tiles, 2);
+      m_block(n_tiles);
       lds_barrier();
     }
   } else {
@@ -1312,7 +1288,7 @@ void launch_prefill_w8(PrefillParams p, hipStream_t stream) {
   static bool attr_set = false;  // benign race: setting twice is harmless
   auto kernel = prefill_varlen_w8_kernel<T, HDP, MODE>;
   constexpr size_t lds_bytes = MODE >= W8_PAGED_DMA ? (size_t)5 * 2 * BN * HDP * 2
-                               : MODE == W8_ROWS   ? (size_t)4 * (BN * HDP + TileW8<HDP>::V_ELEMS) * 2
+                               : MODE == W8_ROWS   ? (size_t)5 * 2 * BN * HDP * 2
                                                    : TileW8<HDP>::LDS_BYTES;
   if (!attr_set) {
     HA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
