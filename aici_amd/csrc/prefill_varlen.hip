@@ -67,9 +67,16 @@ __device__ long long g_phase_trace[64 * 8 * 8];
   do {                                                                                                           \
     if (blockIdx.x == HIPATTN_PHASE_TRACE && j < 64 && lane == 0) g_phase_trace[(j * 8 + wave) * 8 + (slot)] = wall_clock64(); \
   } while (0)
+#define PHASE_MARK(slot)                                                                                        \
+  do {                                                                                                           \
+    if (blockIdx.x == HIPATTN_PHASE_TRACE && (threadIdx.x & 63) == 0) g_phase_trace[(63 * 8 + (threadIdx.x >> 6)) * 8 + (slot)] = wall_clock64(); \
+  } while (0)
 #else
 #define PHASE_STAMP(slot) \
   do {                    \
+  } while (0)
+#define PHASE_MARK(slot) \
+  do {                   \
   } while (0)
 #endif
 
@@ -130,6 +137,7 @@ struct Mfma32<bf16_t> {
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 
 // max(a, b, c) in one instruction.  Scores are never NaN here, so the
 // canonicalising copies fmaxf would add to every MFMA result are not needed.
@@ -498,6 +506,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T *smem = reinterpret_cast<T *>(smem_raw);
+  PHASE_MARK(0);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -553,31 +562,24 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   // 16 bytes per row, 4 rows per instruction) and turned through a private piece of LDS buffers 1 and 2,
   // which no tile reaches before the first barrier.
   constexpr int QSTR = HDP + 8;  // row pitch of the turned Q tile, elements
-  constexpr bool Q_VIA_LDS = (size_t)8 * 32 * QSTR <= (size_t)(NST - 1) * STAGE_ELEMS;
+  // The alternating-block forms turn Q through stages 2.., so that tiles 0 and 1 can be on their way meanwhile.
+  constexpr int Q_STAGE0 = PINGPONG ? 2 : 1;
+  constexpr bool Q_VIA_LDS = (size_t)8 * 32 * QSTR <= (size_t)(NST - Q_STAGE0) * STAGE_ELEMS;
+  constexpr int CPRQ = HDP / 8;
+  constexpr int NQL = (32 * CPRQ + 63) / 64;
   vec8 qreg[KSTEPS];
-  auto load_q = [&]() {
+  u32x4_t qraw[Q_VIA_LDS ? NQL : 1];
+  // The loads of Q (the workgroup's longest wait: nothing else has touched these rows) ...
+  auto q_issue = [&]() {
     if constexpr (Q_VIA_LDS) {
-      constexpr int CPRQ = HDP / 8;
-      constexpr int NQL = (32 * CPRQ + 63) / 64;
-      T *qst = smem + STAGE_ELEMS + wave * (32 * QSTR);
-      u32x4_t raw[NQL];
 #pragma unroll
       for (int it = 0; it < NQL; it++) {
         const int idx = min(it * 64 + lane, 32 * CPRQ - 1);
         const int r = idx / CPRQ, ch = idx % CPRQ;
         const int row = min(wave_row0 + r, Lq - 1);
-        raw[it] = u32x4_t{0u, 0u, 0u, 0u};
-        if (ch < d_chunks) raw[it] = *reinterpret_cast<const u32x4_t *>(qp + (int64_t)row * p.q_row + ch * 8);
+        qraw[it] = u32x4_t{0u, 0u, 0u, 0u};
+        if (ch < d_chunks) qraw[it] = *reinterpret_cast<const u32x4_t *>(qp + (int64_t)row * p.q_row + ch * 8);
       }
-#pragma unroll
-      for (int it = 0; it < NQL; it++) {
-        const int idx = it * 64 + lane;
-        if ((32 * CPRQ) % 64 == 0 || idx < 32 * CPRQ)
-          *reinterpret_cast<u32x4_t *>(qst + (idx / CPRQ) * QSTR + (idx % CPRQ) * 8) = raw[it];
-      }
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ks++)
-        qreg[ks] = *reinterpret_cast<const vec8 *>(qst + c * QSTR + (2 * ks + g) * 8);
     } else {
       const int row = min(wave_row0 + c, Lq - 1);
 #pragma unroll
@@ -588,6 +590,25 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         qreg[ks] = bit_cast<vec8>(raw);
       }
     }
+  };
+  // ... and their way through LDS into the operand registers.
+  auto q_finish = [&]() {
+    if constexpr (Q_VIA_LDS) {
+      T *qst = smem + Q_STAGE0 * STAGE_ELEMS + wave * (32 * QSTR);
+#pragma unroll
+      for (int it = 0; it < NQL; it++) {
+        const int idx = it * 64 + lane;
+        if ((32 * CPRQ) % 64 == 0 || idx < 32 * CPRQ)
+          *reinterpret_cast<u32x4_t *>(qst + (idx / CPRQ) * QSTR + (idx % CPRQ) * 8) = qraw[it];
+      }
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++)
+        qreg[ks] = *reinterpret_cast<const vec8 *>(qst + c * QSTR + (2 * ks + g) * 8);
+    }
+  };
+  auto load_q = [&]() {
+    q_issue();
+    q_finish();
   };
   f32x16_t acc[NDT];
 #pragma unroll
@@ -697,7 +718,11 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     const int idx = (tile & 15) * 4 + dma_r;
     const unsigned lo = __builtin_amdgcn_readlane((int)(uint32_t)tbl_off, idx);
     const unsigned hi = __builtin_amdgcn_readlane((int)(uint32_t)(tbl_off >> 32), idx);
-    const char *src = dma_base + (((uint64_t)hi << 32) | lo);
+    // (an "s" operand is not made a scalar for the asm when the compiler holds the value in vector registers)
+    const uint64_t src_v = reinterpret_cast<uint64_t>(dma_base) + (((uint64_t)hi << 32) | lo);
+    const char *src = reinterpret_cast<const char *>(
+        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(src_v >> 32)) << 32) |
+        (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src_v));
     // the instruction's offset field moves both ends of the copy: the address in memory and the one in LDS
     const unsigned dst = (unsigned)__builtin_amdgcn_readfirstlane(
         (int)(lds0 + (unsigned)(((tile % NST) * STAGE_ELEMS + dma_v * K_ELEMS + dma_r * BLK_ELEMS) * (int)sizeof(T))));
@@ -881,34 +906,36 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   };
   auto store_tile = [&](int stage) { store_tile_paged(stage); };
 
+  // A workgroup has the compute unit to itself, so what it waits for here nobody fills: the loads of Q go
+  // out first (nothing else has touched these rows: the longest wait), the block ids and tiles 0 and 1
+  // behind them, and Q is turned through stages 2.. while the tiles fly.
+  if constexpr (PINGPONG) q_issue();
   if (PAGED && n_tiles > 0) tbl_cur = load_ids(0);
   if constexpr (DMA) {
     tbl_off = ids_to_offsets(tbl_cur);
-    // Tile 0 flies into stage 0 while Q is turned through stages 1..3; tiles 1 and 2 follow once every
-    // wavefront has its Q.
+    PHASE_MARK(4);
     if (n_tiles > 0) dma_tile(0);
-    clear_image_tails(0, 0);
-    load_q();
-    if (n_tiles > 0) dma_wait(0, false);
-    __syncthreads();
     if (n_tiles > 1) dma_tile(1);
+    clear_image_tails(0, 1);
+    q_finish();
+    PHASE_MARK(5);
+    if (n_tiles > 0) dma_wait(0, n_tiles > 1);
+    __syncthreads();
+    PHASE_MARK(6);
     if (n_tiles > 2) dma_tile(2);
-    clear_image_tails(1, NST - 1);  // seen by all after the barrier in front of the loop; stage 1 is first read there
+    clear_image_tails(2, NST - 1);  // seen by all after the barrier in front of the loop
   } else if constexpr (ROWS) {
-    // Tile 0 arrives in stage 0 while Q is turned through stages 1..3; then K of tiles 1 and 2 is copied,
-    // V of tile 1 goes through the registers into its stage and V of tile 2 into the registers.
+    // V of tile 0 goes through the registers into its stage; after the barrier V of tile 1 is asked for.
     if (n_tiles > 0) {
       load_v_rows(0);
       k_rows_dma(0);
     }
-    load_q();
+    if (n_tiles > 1) k_rows_dma(1);
+    q_finish();
     if (n_tiles > 0) store_v_rows(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (n_tiles > 1) {
-      load_v_rows(1);
-      k_rows_dma(1);
-    }
+    if (n_tiles > 1) load_v_rows(1);
     if (n_tiles > 2) k_rows_dma(2);
   } else {
     if (n_tiles > 0) load_tile(0);
@@ -965,7 +992,11 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     }
   };
   // Tiles entirely past the diagonal of every row of this wavefront are skipped.
-  auto skip_tile = [&](int j) { return (wave_row0 >= Lq) || (p.causal && j * BN > wave_last_row + off); };
+  // Rows form: the wavefront's first row as a scalar, so that the tests on it run in the scalar unit and hold no
+  // vector register (the register had been spilled, and its reload at the top of every tile waited for the
+  // copies in flight).  The other forms allocate worse with it.
+  const int wave_row0_u = ROWS ? __builtin_amdgcn_readfirstlane(wave_row0) : wave_row0;
+  auto skip_tile = [&](int j) { return (wave_row0_u >= Lq) || (p.causal && j * BN > wave_row0_u + 31 + off); };
 
   // ---- the pipelined tile loop (staged tiles; block images run the alternating blocks further down) ----
   // Iteration j of a wavefront: the matrix pipe computes S(j+1) = K(j+1).Q^T while
@@ -979,6 +1010,11 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   constexpr int EXPS = NQ - MAXS;  // the rest the exponentials
   constexpr int QK_DEPTH = 3;      // K operands read ahead of their MFMA
 
+  // (not in the rows form: it has no register to spare, and a reload from scratch inside the loop waits for
+  // every copy in flight)
+  constexpr bool SPEC = DMA;
+  bool seeded = false;  // every row of this wavefront has a finite reference maximum
+  const float spec_limit = fast_exp2(p.rescale_thr);
   // DO_QK: S(j+1) is wanted (written to sn); the softmax of S(j) (in s) always runs.
   auto qk_softmax = [&](auto do_qk, int j, f32x16_t(&s)[2], f32x16_t(&sn)[2], vec8(&pk)[2][2]) {
     constexpr bool DO_QK = decltype(do_qk)::value;
@@ -1001,9 +1037,9 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       }
     };
 
-    const bool need_mask = (k0 + BN > Lk) || (p.causal && k0 + BN - 1 > wave_row0 + off);
+    const bool need_mask = (k0 + BN > Lk) || (p.causal && k0 + BN - 1 > wave_row0_u + off);
     if (need_mask) {
-      const int row = wave_row0 + c;
+      const int row = wave_row0_u + c;
       int limit = p.causal ? row + off : Lk - 1;
       limit = min(limit, Lk - 1);
 #pragma unroll
@@ -1015,6 +1051,33 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
           if (key > limit) s[kt][i] = -INFINITY;
         }
     }
+    // Block images: once every row has a finite reference maximum, a tile without masked keys is first tried
+    // against that reference as it stands, without looking for the row maximum.  A lane whose sum of
+    // probabilities exceeds the rescale threshold may hold a probability above it: then the tile is done
+    // again the exact way, which also moves the reference to the new maximum, so that the next tiles pass.
+    // When the try passes, the exact way would have given the same probabilities and (but for the order of
+    // the additions) the same sums.
+    bool retry = false;
+    if constexpr (SPEC && !DO_QK) {
+      if (seeded && !need_mask) {
+        float psum = 0.f, psum2 = 0.f;
+#pragma unroll
+        for (int v = 0; v < 32; v += 2) {
+          const float e0 = fast_exp2(s[v / 16][v % 16] * p.scale_log2 - m_run);
+          const float e1 = fast_exp2(s[v / 16][v % 16 + 1] * p.scale_log2 - m_run);
+          pk[v / 16][(v % 16) / 8][v % 8] = from_float<T>(e0);
+          pk[v / 16][(v % 16) / 8][v % 8 + 1] = from_float<T>(e1);
+          psum += e0;
+          psum2 += e1;
+        }
+        psum += psum2;
+        if (__builtin_expect(!__any(psum > spec_limit), 1)) {
+          l_run += psum;
+          return;
+        }
+        retry = true;
+      }
+    }
     // row maximum in the shadow of the first MAXS MFMAs
     float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
@@ -1025,7 +1088,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         if (i > 0) mx = max3(mx, s[0][i], s[1][i]);
     }
     mx = max_across_halves(mx) * p.scale_log2;
-    const bool grow = mx > m_run + p.rescale_thr;
+    const bool grow = mx > m_run + (retry ? 0.f : p.rescale_thr);
     if (__builtin_expect(__any(grow), 0)) {
       const float m_new = grow ? mx : m_run;
       const float alpha = grow ? fast_exp2(m_run - m_new) : 1.0f;
@@ -1034,6 +1097,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       for (int dt = 0; dt < NDT; dt++) acc[dt] *= alpha;
       m_run = m_new;
     }
+    if constexpr (SPEC && !DO_QK) seeded = !__any(m_run == -INFINITY);
     const float msub = m_run == -INFINITY ? 0.f : m_run;
     const float pmax = fast_exp2(mx - msub);
     float psum = g == 0 ? to_float(from_float<T>(pmax)) - pmax : 0.f;
@@ -1103,7 +1167,9 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     auto v_block = [&](int t) {
       if (!skip_tile(t)) qk_softmax(std::false_type{}, t, s_a, s_b, pk);
       if constexpr (DMA) {
+        { const int j = t; PHASE_STAMP(4); }
         if (t + 2 < n_tiles) dma_wait(t + 2, false);
+        { const int j = t; PHASE_STAMP(5); }
         if (t + 3 < n_tiles) dma_tile(t + 3);
       } else {
         // K of tile t + 2 has landed (its V went into LDS behind the last M block)
@@ -1120,6 +1186,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     const bool second_group = wave_u >= 4;
     if constexpr (DMA) {
       if (!second_group) m_block(0);
+      PHASE_MARK(7);
       if (n_tiles > 1) dma_wait(1, n_tiles > 2);
     } else {
       if (n_tiles > 1) {
@@ -1130,7 +1197,12 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       if (!second_group) m_block(0);  // its tail stores V of tile 2; the other group's M(0) does so in period 0
     }
     lds_barrier();
+    PHASE_MARK(1);
     if (!second_group) {
+      // The loop starts on a 64-byte boundary: where it happens to fall otherwise moves the time of this
+      // kernel by several per cent from one build to the next (1.09 against 1.03 ms on 8 x 4096 tokens for
+      // the same instructions at another address).
+      asm volatile(".p2align 6");
       for (int j = 0; j < n_tiles; j++) {
         PHASE_STAMP(0);
         v_block(j);
@@ -1141,6 +1213,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       }
       lds_barrier();  // the other group's last product still reads its tile
     } else {
+      asm volatile(".p2align 6");
       for (int j = 0; j < n_tiles; j++) {
         PHASE_STAMP(0);
         m_block(j);
@@ -1214,6 +1287,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     }
   }
 
+  PHASE_MARK(2);
   // ---- epilogue ---------------------------------------------------------------
   // The accumulators hold O^T: a lane has 4 consecutive head elements of one row per register quad,
   // which stored directly would be 16-byte pieces of 32 rows per instruction.  Each wavefront turns
@@ -1281,6 +1355,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     const float lse = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : INFINITY;
     p.lse[((int64_t)b * p.Hq + h_e) * p.lse_pitch + wave_row0_e + c_e] = lse;
   }
+  PHASE_MARK(3);
 }
 
 template <typename T, int HDP, int MODE = W8_ROWS>

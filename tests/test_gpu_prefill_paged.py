@@ -86,6 +86,41 @@ def test_matches_oracle(device, dtype, heads):
     assert (got.float() - want).abs().max().item() <= TOL[dtype]
 
 
+@pytest.mark.parametrize("slope", [6.0, 0.5, -6.0])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_scores_that_drift_along_the_keys(device, dtype, slope):
+    """The scores of every row rise (or fall) steadily with the key's position: by `slope` powers of two per
+    64-key tile.  Rising fast, the running reference maximum of a row is outgrown every tile or two -- the
+    case in which a tile tried against the old reference has to be done again; rising slowly, it is outgrown
+    only every sixteen tiles; falling, never after the first tile."""
+    Hq, Hkv, d = 8, 2, 128
+    c = paged_case(36, [(1500, 520), (0, 700)], Hq, Hkv, d, dtype, 200)
+    g = torch.Generator().manual_seed(37)
+    u = torch.nn.functional.normalize(torch.randn(d, generator=g), dim=0)
+    # q . k * scale * log2(e) = drift(j) + noise, drift(j) = slope * j / 64
+    c["q"] = (0.3 * torch.randn(c["q"].shape, generator=g) + 4.0 * u).to(dtype)
+    kc, vc = c["kc"], c["vc"]
+    for i, lk in enumerate(c["lens_k"]):
+        j = torch.arange(lk, dtype=torch.float32)
+        along = slope * j / 64.0 / (4.0 * c["scale"] * math.log2(math.e))
+        k = (0.3 * torch.randn((lk, Hkv, d), generator=g) + along[:, None, None] * u).to(dtype)
+        v = torch.randn((lk, Hkv, d), generator=g).to(dtype)
+        ref.reshape_and_cache(k, v, kc, vc, c["slots"][i])
+    got, lse = run_paged(c, device, lse=True)
+    want = oracle(c, Hq, Hkv, d)
+    assert not torch.isnan(got).any()
+    assert (got.cpu().float() - want).abs().max().item() <= TOL[dtype]
+    # the log-sum-exp against the rows form (which never tries a tile against an old reference) on the same K/V
+    gm = torch.cat(c["slots"]).to(torch.int32).to(device)
+    gk = torch.empty((gm.numel(), Hkv, d), dtype=dtype, device=device)
+    gv = torch.empty_like(gk)
+    K.gather_cached_kv(gk, gv, kc.to(device), vc.to(device), gm)
+    _, lse2 = K.flash_attn_varlen(c["q"].to(device), gk, gv, c["cu_q"].to(device), W.offsets(c["lens_k"]).to(device),
+                                  max(c["lens_q"]), max(c["lens_k"]), c["scale"], True, return_lse=True)
+    for i, lq in enumerate(c["lens_q"]):
+        assert torch.allclose(lse[i, :, :lq], lse2[i, :, :lq], atol=2e-3, rtol=1e-4)
+
+
 def test_agrees_with_gather_then_contiguous_prefill_and_lse(device):
     dtype = torch.bfloat16
     Hq, Hkv, d = 32, 8, 128
