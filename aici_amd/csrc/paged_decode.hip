@@ -633,6 +633,8 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void paged_decode_flat_kern
       if (HD <= 128) {
         PairRegs<HD> ra, rb;
         issue(0, ra);
+        // the loop on a 256-byte boundary: 1 % on the whole step against where it happened to fall
+        asm volatile(".p2align 8");
         for (int it = 0; it < nsub; it += 2) {
           if (it + 1 < nsub) issue(it + 1, rb);
           fold(it, ra);

@@ -145,6 +145,14 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // operations only.  __syncthreads() also drains the vector-memory counter,
 // which would make every tile wait for the global loads of the tile after next
 // that were just issued.
+// A pointer that is the same in every lane, as the scalar it is: an "s" operand of inline asm is not made one
+// when the compiler holds the value in vector registers.
+template <typename P>
+__device__ __forceinline__ const P *uniform_ptr(const P *ptr) {
+  const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+  return reinterpret_cast<const P *>(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32)) << 32) |
+                                     (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v));
+}
 __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
@@ -480,8 +488,9 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   constexpr bool ROWS = MODE == W8_ROWS;
   constexpr bool DMA = MODE == W8_PAGED_DMA || MODE == W8_PAGED_DMA_PART;
   // W8_ROWS: K tiles are copied global -> LDS into the layout of the cache's block images (16-byte runs of a
-  // row of k are the images' units, so a lane address per run is all it takes), V tiles are transposed
-  // through registers.  Both forms run the alternating MFMA / softmax blocks.
+  // row of k are the images' units, so a lane address per run is all it takes); V tiles are copied as the
+  // rows they are and the second product reads its operands from them with the transposing LDS read.  Both
+  // forms run the alternating MFMA / softmax blocks.
   constexpr bool KIMG = DMA || ROWS;      // K tiles lie in LDS as block images
   constexpr bool PINGPONG = DMA || ROWS;
   // W8_PAGED_DMA_PART: head sizes below HDP (Phi-2's 80 in the 96-wide instance).  An image then fills only the
@@ -490,8 +499,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   constexpr bool DMA_PART = MODE == W8_PAGED_DMA_PART;
   // W8_PAGED_DMA keeps a tile as the four block images of the cache, unpadded, in four stages.
   // Block images and rows: five stages (all of the 160 KB at head size 128) and one barrier per tile; staged:
-  // three.  For five to fit, the V^T tiles of the rows form are not padded but swizzled: the 16-byte run q of
-  // row r lies at run q ^ ((r >> 1) & 7), which keeps the operand reads free of bank conflicts.
+  // three.  No tile is padded; where reads would collide, runs change places within their row (see v_rows_dma).
   constexpr int NST = PINGPONG ? 5 : 3;
   constexpr int K_ELEMS = KIMG ? BN * HDP : TL::K_ELEMS;
   constexpr int STAGE_ELEMS = PINGPONG ? 2 * BN * HDP : K_ELEMS + TL::V_ELEMS;
@@ -500,9 +508,6 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   constexpr int CPR = HDP / 8;                // 16-byte chunks per K row
   constexpr int K_CHUNKS = BN * CPR;          // per tile
   constexpr int NLOADK = (K_CHUNKS + 511) / 512;
-  constexpr int V_ITEMS = 16 * (HDP / 4);     // (4 keys) x (4 head elements) blocks per tile
-  constexpr int NLOADV = (V_ITEMS + 511) / 512;
-  static_assert(NLOADV == 1, "one (4 keys x 4 elements) block per thread");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T *smem = reinterpret_cast<T *>(smem_raw);
@@ -618,22 +623,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   float m_run = -INFINITY, l_run = 0.f;
 
   // ---- tile staging ---------------------------------------------------------
-  // K: chunk (t + 512 i) of the tile, row-major.  V: thread t owns the block of
-  // 4 keys x 4 head elements (kg4, dg); it loads 4 x 8 B, transposes in
-  // registers and writes 4 x 8 B, one per head element, into V^T.  Within a
-  // wavefront 8 lanes cover 8 consecutive dg (64 B of a global row) and 8 lane
-  // groups cover 8 consecutive kg4, which keeps the transposed writes at a
-  // 2-way bank conflict.  Addresses are clamped, never predicated: keys past Lk
-  // re-read the last key (masked later), head elements past d re-read the last
-  // real ones (never stored).
   u32x4_t kst[NLOADK];
-  u32x2_t vst[NLOADV][4];
-  const int v_dg = (wave & 3) * 8 + (lane & 7);        // 4-element group of the head dimension
-  const int v_kg4 = (wave >> 2) * 8 + (lane >> 3);     // 4-key group of the tile, 0..15
-  // Per-thread byte offsets inside a tile, relative to its first key, in 32
-  // bits (the launcher checks that 64 rows fit): a full tile's loads are then
-  // a uniform base plus a 32-bit lane offset.
-  const uint32_t v_boff = (uint32_t)(((int64_t)(v_kg4 * 4) * p.v_row + min(v_dg, p.d / 4 - 1) * 4) * (int64_t)sizeof(T));
   // PAGED: blocks of the cache instead of rows of k / v.  A tile is 4 blocks; threads follow the cache's
   // own order so that consecutive lanes read consecutive 16-byte runs: K unit u = (block, chunk c8,
   // token) is the run [c8][token] of its block and lands in LDS row 16*block + token; V unit u = (block,
@@ -795,22 +785,6 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       }
     }
   };
-  // W8_ROWS, V: thread t's block of 4 keys x 4 head elements of the tile.
-  auto load_v_rows = [&](int tile) {
-    const int k0 = tile * BN;
-    if (k0 + BN <= Lk) {
-      const char *vt = reinterpret_cast<const char *>(vp + (int64_t)k0 * p.v_row);
-#pragma unroll
-      for (int kk = 0; kk < 4; kk++)
-        vst[0][kk] = *reinterpret_cast<const u32x2_t *>(vt + (int64_t)kk * p.v_row * (int64_t)sizeof(T) + v_boff);
-    } else {  // the last, partial tile: clamp every key to the last real one
-#pragma unroll
-      for (int kk = 0; kk < 4; kk++) {
-        const int key = min(k0 + v_kg4 * 4 + kk, Lk - 1);
-        vst[0][kk] = *reinterpret_cast<const u32x2_t *>(vp + (int64_t)key * p.v_row + min(v_dg, p.d / 4 - 1) * 4);
-      }
-    }
-  };
   // W8_ROWS, K: the tile goes global -> LDS in 1 KiB pieces, 4 x HDP / 32 of them, dealt round the
   // wavefronts.  Piece q is runs [4 pi .. 4 pi + 4) x 16 tokens of block r = q / (HDP / 32), pi = q %
   // (HDP / 32), of the image layout [run][token][8 elements]: lane l fetches run 4 pi + l / 16 of token
@@ -837,9 +811,56 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
           off = (uint32_t)(((int64_t)(key - k0) * p.k_row + (min(4 * pi + kd_run, d_chunks - 1) - 4 * pi) * 8) * (int64_t)sizeof(T));
           first = (int64_t)k0 * p.k_row + 32 * pi;
         }
-        const T *src = kp + first;
+        const T *src = uniform_ptr(kp + first);
         const unsigned dst = (unsigned)__builtin_amdgcn_readfirstlane(
             (int)(lds_base + (unsigned)(((tile % NST) * STAGE_ELEMS + r * (HDP * 16)) * (int)sizeof(T)) + pi * 1024));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(dst), "v"(off), "s"(src)
+                     : "memory", "m0");
+      }
+    }
+  };
+  // W8_ROWS, V: the tile's rows go global -> LDS as they are, [key][HDP elements], in 1 KiB pieces (64 16-byte
+  // runs in row order) dealt round the wavefronts; the second product reads its operands from them with the
+  // transposing LDS read.  For those reads to be free of bank conflicts -- one covers 64 bytes of each of 4
+  // consecutive rows -- run c of row r lies at run c ^ vswz(r) of its row where the row pitch is a multiple of
+  // 256 bytes (64-byte groups of runs change places, by the row's low bits); a lane's place in LDS is given by
+  // the instruction, so it fetches the run that belongs there.  Runs past d fetch the last real one (rows of the
+  // output nobody stores), keys past Lk the last real key (their probabilities are zero).
+  constexpr int CPRV = HDP / 8;          // runs per row
+  constexpr int VNP = BN * CPRV / 64;    // pieces per tile
+  constexpr int VNPW = (VNP + 7) / 8;    // ... per wavefront
+  auto vswz = [](int r) -> int { return HDP == 128 ? (r & 3) << 2 : (HDP == 64 ? ((r >> 1) & 1) << 2 : 0); };
+  uint32_t vd_off[VNPW];
+  if constexpr (ROWS) {
+#pragma unroll
+    for (int i = 0; i < VNPW; i++) {
+      const int u = (wave + 8 * i) * 64 + lane;  // the lane's run of the tile, in LDS order
+      const int r = u / CPRV, pc = u % CPRV;
+      vd_off[i] = (uint32_t)(((int64_t)r * p.v_row + min(pc ^ vswz(r), d_chunks - 1) * 8) * (int64_t)sizeof(T));
+    }
+  }
+  auto v_rows_dma = [&](int tile) {
+    const int k0 = tile * BN;
+    const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem_raw;
+    const T *src = uniform_ptr(vp + (int64_t)k0 * p.v_row);
+#pragma unroll
+    for (int i = 0; i < VNPW; i++) {
+      const int q = wave_u + 8 * i;
+      if (VNP % 8 == 0 || q < VNP) {
+        uint32_t off = vd_off[i];
+        if (k0 + BN > Lk) {
+          // (the lane number through an opaque copy: hoisted out of the loop, what is derived from it here
+          // would hold registers that the loop does not have)
+          int l2 = lane;
+          asm volatile("" : "+v"(l2));
+          const int u = q * 64 + l2;
+          const int r = u / CPRV, pc = u % CPRV;
+          off = (uint32_t)(((int64_t)(min(k0 + r, Lk - 1) - k0) * p.v_row + min(pc ^ vswz(r), d_chunks - 1) * 8) * (int64_t)sizeof(T));
+        }
+        const unsigned dst = (unsigned)__builtin_amdgcn_readfirstlane(
+            (int)(lds_base + (unsigned)(((tile % NST) * STAGE_ELEMS + K_ELEMS) * (int)sizeof(T)) + q * 1024));
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                      :
                      : "s"(dst), "v"(off), "s"(src)
@@ -884,26 +905,6 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       }
     }
   };
-  // W8_ROWS, V: the thread's block transposed in registers and written into V^T, keys in their own order (the
-  // order in which the image layout of K hands the scores to the second product).
-  auto store_v_rows = [&](int stage) {
-    T *vs = smem + stage * STAGE_ELEMS + K_ELEMS;
-    if (V_ITEMS % 512 == 0 || v_dg < HDP / 4) {
-      // 4x4 transpose of 16-bit values: out[dd] = {k0.d, k1.d, k2.d, k3.d}
-      const unsigned a0 = vst[0][0][0], a1 = vst[0][0][1], b0 = vst[0][1][0], b1 = vst[0][1][1];
-      const unsigned c0 = vst[0][2][0], c1 = vst[0][2][1], e0 = vst[0][3][0], e1 = vst[0][3][1];
-      u32x2_t o[4];
-      o[0] = u32x2_t{__builtin_amdgcn_perm(b0, a0, 0x05040100u), __builtin_amdgcn_perm(e0, c0, 0x05040100u)};
-      o[1] = u32x2_t{__builtin_amdgcn_perm(b0, a0, 0x07060302u), __builtin_amdgcn_perm(e0, c0, 0x07060302u)};
-      o[2] = u32x2_t{__builtin_amdgcn_perm(b1, a1, 0x05040100u), __builtin_amdgcn_perm(e1, c1, 0x05040100u)};
-      o[3] = u32x2_t{__builtin_amdgcn_perm(b1, a1, 0x07060302u), __builtin_amdgcn_perm(e1, c1, 0x07060302u)};
-#pragma unroll
-      for (int dd = 0; dd < 4; dd++) {
-        const int r = v_dg * 4 + dd;
-        *reinterpret_cast<u32x2_t *>(vs + r * BN + (((v_kg4 >> 1) ^ ((r >> 1) & 7)) * 8) + (v_kg4 & 1) * 4) = o[dd];
-      }
-    }
-  };
   auto store_tile = [&](int stage) { store_tile_paged(stage); };
 
   // A workgroup has the compute unit to itself, so what it waits for here nobody fills: the loads of Q go
@@ -925,18 +926,21 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     if (n_tiles > 2) dma_tile(2);
     clear_image_tails(2, NST - 1);  // seen by all after the barrier in front of the loop
   } else if constexpr (ROWS) {
-    // V of tile 0 goes through the registers into its stage; after the barrier V of tile 1 is asked for.
     if (n_tiles > 0) {
-      load_v_rows(0);
       k_rows_dma(0);
+      v_rows_dma(0);
     }
-    if (n_tiles > 1) k_rows_dma(1);
+    if (n_tiles > 1) {
+      k_rows_dma(1);
+      v_rows_dma(1);
+    }
     q_finish();
-    if (n_tiles > 0) store_v_rows(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (n_tiles > 1) load_v_rows(1);
-    if (n_tiles > 2) k_rows_dma(2);
+    if (n_tiles > 2) {
+      k_rows_dma(2);
+      v_rows_dma(2);
+    }
   } else {
     if (n_tiles > 0) load_tile(0);
     load_q();
@@ -956,11 +960,16 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   const int k_lane_off = KIMG ? (c >> 4) * (HDP * 16) + g * 128 + (((c >> 2) & 1) * 8 + ((c >> 3) & 1) * 4 + (c & 3)) * 8
                               : c * TL::KSTR + g * 8;
   const int v_lane_off = DMA ? g * 256 + c * 8 : c * TL::VTSTR + g * 8;
-  // W8_ROWS: element offset of run 2 ks + g of this lane's V^T row within a 32-row block, for the four
-  // contraction steps ks of a tile (the swizzle is the same in every block: 32 rows are a multiple of 16)
-  int v_swz_off[4];
+  // W8_ROWS: the transposing read hands lane (g, rh, li) head element 16 rh + li of the 4 keys whose rows its
+  // 16-lane group addresses -- source lane s gives 8 bytes of row s / 4: elements 4 (s % 4) .. + 4 of the
+  // 16 -- so two reads, at rows 8 g + s / 4 and 4 further, make the 8 keys of a P.V operand.  Element offset
+  // of the lane's 8 bytes for output tile dt, first 16-key step:
+  int vtr_off[NDT];
 #pragma unroll
-  for (int ks = 0; ks < 4; ks++) v_swz_off[ks] = c * BN + (((2 * ks + g) ^ ((c >> 1) & 7)) * 8);
+  for (int dt = 0; dt < NDT; dt++) {
+    const int li = lane & 15, rh = (lane >> 4) & 1, r = 8 * g + (li >> 2);
+    vtr_off[dt] = r * HDP + ((dt * 4 + 2 * rh + ((li & 3) >> 1)) ^ vswz(r)) * 8 + 4 * (li & 1);
+  }
   constexpr int K_HALF = KIMG ? 2 * HDP * 16 : 32 * TL::KSTR;  // elements between the two 32-key halves of a K tile
   constexpr int K_STEP = KIMG ? 256 : 16;                      // ... between contraction steps (16 head elements)
   const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -992,11 +1001,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     }
   };
   // Tiles entirely past the diagonal of every row of this wavefront are skipped.
-  // Rows form: the wavefront's first row as a scalar, so that the tests on it run in the scalar unit and hold no
-  // vector register (the register had been spilled, and its reload at the top of every tile waited for the
-  // copies in flight).  The other forms allocate worse with it.
-  const int wave_row0_u = ROWS ? __builtin_amdgcn_readfirstlane(wave_row0) : wave_row0;
-  auto skip_tile = [&](int j) { return (wave_row0_u >= Lq) || (p.causal && j * BN > wave_row0_u + 31 + off); };
+  auto skip_tile = [&](int j) { return (wave_row0 >= Lq) || (p.causal && j * BN > wave_last_row + off); };
 
   // ---- the pipelined tile loop (staged tiles; block images run the alternating blocks further down) ----
   // Iteration j of a wavefront: the matrix pipe computes S(j+1) = K(j+1).Q^T while
@@ -1010,11 +1015,6 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   constexpr int EXPS = NQ - MAXS;  // the rest the exponentials
   constexpr int QK_DEPTH = 3;      // K operands read ahead of their MFMA
 
-  // (not in the rows form: it has no register to spare, and a reload from scratch inside the loop waits for
-  // every copy in flight)
-  constexpr bool SPEC = DMA;
-  bool seeded = false;  // every row of this wavefront has a finite reference maximum
-  const float spec_limit = fast_exp2(p.rescale_thr);
   // DO_QK: S(j+1) is wanted (written to sn); the softmax of S(j) (in s) always runs.
   auto qk_softmax = [&](auto do_qk, int j, f32x16_t(&s)[2], f32x16_t(&sn)[2], vec8(&pk)[2][2]) {
     constexpr bool DO_QK = decltype(do_qk)::value;
@@ -1037,9 +1037,9 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       }
     };
 
-    const bool need_mask = (k0 + BN > Lk) || (p.causal && k0 + BN - 1 > wave_row0_u + off);
+    const bool need_mask = (k0 + BN > Lk) || (p.causal && k0 + BN - 1 > wave_row0 + off);
     if (need_mask) {
-      const int row = wave_row0_u + c;
+      const int row = wave_row0 + c;
       int limit = p.causal ? row + off : Lk - 1;
       limit = min(limit, Lk - 1);
 #pragma unroll
@@ -1051,33 +1051,6 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
           if (key > limit) s[kt][i] = -INFINITY;
         }
     }
-    // Block images: once every row has a finite reference maximum, a tile without masked keys is first tried
-    // against that reference as it stands, without looking for the row maximum.  A lane whose sum of
-    // probabilities exceeds the rescale threshold may hold a probability above it: then the tile is done
-    // again the exact way, which also moves the reference to the new maximum, so that the next tiles pass.
-    // When the try passes, the exact way would have given the same probabilities and (but for the order of
-    // the additions) the same sums.
-    bool retry = false;
-    if constexpr (SPEC && !DO_QK) {
-      if (seeded && !need_mask) {
-        float psum = 0.f, psum2 = 0.f;
-#pragma unroll
-        for (int v = 0; v < 32; v += 2) {
-          const float e0 = fast_exp2(s[v / 16][v % 16] * p.scale_log2 - m_run);
-          const float e1 = fast_exp2(s[v / 16][v % 16 + 1] * p.scale_log2 - m_run);
-          pk[v / 16][(v % 16) / 8][v % 8] = from_float<T>(e0);
-          pk[v / 16][(v % 16) / 8][v % 8 + 1] = from_float<T>(e1);
-          psum += e0;
-          psum2 += e1;
-        }
-        psum += psum2;
-        if (__builtin_expect(!__any(psum > spec_limit), 1)) {
-          l_run += psum;
-          return;
-        }
-        retry = true;
-      }
-    }
     // row maximum in the shadow of the first MAXS MFMAs
     float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
@@ -1088,7 +1061,7 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         if (i > 0) mx = max3(mx, s[0][i], s[1][i]);
     }
     mx = max_across_halves(mx) * p.scale_log2;
-    const bool grow = mx > m_run + (retry ? 0.f : p.rescale_thr);
+    const bool grow = mx > m_run + p.rescale_thr;
     if (__builtin_expect(__any(grow), 0)) {
       const float m_new = grow ? mx : m_run;
       const float alpha = grow ? fast_exp2(m_run - m_new) : 1.0f;
@@ -1097,7 +1070,6 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       for (int dt = 0; dt < NDT; dt++) acc[dt] *= alpha;
       m_run = m_new;
     }
-    if constexpr (SPEC && !DO_QK) seeded = !__any(m_run == -INFINITY);
     const float msub = m_run == -INFINITY ? 0.f : m_run;
     const float pmax = fast_exp2(mx - msub);
     float psum = g == 0 ? to_float(from_float<T>(pmax)) - pmax : 0.f;
@@ -1138,29 +1110,57 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       const T *vs_base = smem + (j % NST) * STAGE_ELEMS + K_ELEMS;
       // Step n = (contraction step n / NDT, output tile n % NDT): consecutive MFMAs go to different
       // accumulators, so none waits for the result of the one before it.
-      auto rd = [&](int n) -> vec8 {
-        if constexpr (DMA) return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + (n / NDT) * (HDP * 16) + (n % NDT) * 512);
-        return *reinterpret_cast<const vec8 *>(vs_base + v_swz_off[n / NDT] + (n % NDT) * 32 * BN);
-      };
-      vec8 va[4];
+      if constexpr (DMA) {
+        auto rd = [&](int n) -> vec8 {
+          return *reinterpret_cast<const vec8 *>(vs_base + v_lane_off + (n / NDT) * (HDP * 16) + (n % NDT) * 512);
+        };
+        vec8 va[4];
 #pragma unroll
-      for (int n = 0; n < 3 && n < PV_STEPS; n++) va[n] = rd(n);
+        for (int n = 0; n < 3 && n < PV_STEPS; n++) va[n] = rd(n);
 #pragma unroll
-      for (int n = 0; n < PV_STEPS; n++) {
-        if (n + 3 < PV_STEPS) va[(n + 3) % 4] = rd(n + 3);
-        __builtin_amdgcn_sched_barrier(0);
-        acc[n % NDT] = Mfma32<T>::run(va[n % 4], pk[(n / NDT) / 2][(n / NDT) % 2], acc[n % NDT]);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int n = 0; n < PV_STEPS; n++) {
+          if (n + 3 < PV_STEPS) va[(n + 3) % 4] = rd(n + 3);
+          __builtin_amdgcn_sched_barrier(0);
+          acc[n % NDT] = Mfma32<T>::run(va[n % 4], pk[(n / NDT) / 2][(n / NDT) % 2], acc[n % NDT]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        // Rows: two transposing reads per operand, written as asm -- the builtin takes no offset, and a
+        // register per address is 32 registers -- so the waits for them are written here too (the compiler
+        // does not see these reads; what it waits for on its own account only ever waits longer).
+        unsigned va_addr[NDT];
+        const unsigned vs_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem_raw +
+                                (unsigned)(((j % NST) * STAGE_ELEMS + K_ELEMS) * (int)sizeof(T));
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) va_addr[dt] = vs_lds + (unsigned)(vtr_off[dt] * (int)sizeof(T));
+        u32x2_t lo[4], hi[4];
+        auto rd = [&](int n) {
+          constexpr int ROW4 = 4 * HDP * (int)sizeof(T);
+          asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+                       : "=&v"(lo[n % 4]), "=&v"(hi[n % 4])
+                       : "v"(va_addr[n % NDT]), "n"((n / NDT) * 4 * ROW4), "n"((n / NDT) * 4 * ROW4 + ROW4)
+                       : "memory");
+        };
+#pragma unroll
+        for (int n = 0; n < 3 && n < PV_STEPS; n++) rd(n);
+#pragma unroll
+        for (int n = 0; n < PV_STEPS; n++) {
+          if (n + 3 < PV_STEPS) {
+            rd(n + 3);
+            asm volatile("s_waitcnt lgkmcnt(6)" ::: "memory");
+          } else {
+            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(2 * (PV_STEPS - 1 - n)) : "memory");
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          const u32x4_t av = {lo[n % 4][0], lo[n % 4][1], hi[n % 4][0], hi[n % 4][1]};
+          acc[n % NDT] = Mfma32<T>::run(bit_cast<vec8>(av), pk[(n / NDT) / 2][(n / NDT) % 2], acc[n % NDT]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     };
-    // W8_ROWS: the V rows that this wavefront asked for in its last V block (tile t + 2) are transposed and
-    // stored behind the MFMAs, where the wavefront would otherwise wait at the barrier.
     auto m_block = [&](int t) {
       if (t >= 1 && !skip_tile(t - 1)) pv_images(t - 1);
       if (t < n_tiles && !skip_tile(t)) phase_qk(t % NST, s_a);
-      if constexpr (ROWS) {
-        if (t + 2 < n_tiles) store_v_rows((t + 2) % NST);
-      }
     };
     // After the softmax: this wavefront's part of tile t + 2, sent a period ago, is waited for, and its part of
     // tile t + 3 follows.
@@ -1172,13 +1172,10 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         { const int j = t; PHASE_STAMP(5); }
         if (t + 3 < n_tiles) dma_tile(t + 3);
       } else {
-        // K of tile t + 2 has landed (its V went into LDS behind the last M block)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        // The loads first: the compiler counts only its own memory operations when it places waits, and a
-        // wait it puts between these loads would otherwise also wait for the copies just issued.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's pieces of tile t + 2
         if (t + 3 < n_tiles) {
-          load_v_rows(t + 3);
           k_rows_dma(t + 3);
+          v_rows_dma(t + 3);
         }
       }
     };
@@ -1189,12 +1186,8 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
       PHASE_MARK(7);
       if (n_tiles > 1) dma_wait(1, n_tiles > 2);
     } else {
-      if (n_tiles > 1) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        store_v_rows(1);
-      }
-      if (n_tiles > 2) load_v_rows(2);
-      if (!second_group) m_block(0);  // its tail stores V of tile 2; the other group's M(0) does so in period 0
+      if (!second_group) m_block(0);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // tiles 1 and 2
     }
     lds_barrier();
     PHASE_MARK(1);

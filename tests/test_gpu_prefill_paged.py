@@ -90,9 +90,9 @@ def test_matches_oracle(device, dtype, heads):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_scores_that_drift_along_the_keys(device, dtype, slope):
     """The scores of every row rise (or fall) steadily with the key's position: by `slope` powers of two per
-    64-key tile.  Rising fast, the running reference maximum of a row is outgrown every tile or two -- the
-    case in which a tile tried against the old reference has to be done again; rising slowly, it is outgrown
-    only every sixteen tiles; falling, never after the first tile."""
+    64-key tile.  Rising fast, the reference maximum of a row (moved only when outgrown by 2^8) moves every
+    tile or two and the accumulators are rescaled each time; rising slowly, every sixteen tiles, with
+    probabilities up to 256 in between; falling, never after the first tile."""
     Hq, Hkv, d = 8, 2, 128
     c = paged_case(36, [(1500, 520), (0, 700)], Hq, Hkv, d, dtype, 200)
     g = torch.Generator().manual_seed(37)
@@ -110,7 +110,7 @@ def test_scores_that_drift_along_the_keys(device, dtype, slope):
     want = oracle(c, Hq, Hkv, d)
     assert not torch.isnan(got).any()
     assert (got.cpu().float() - want).abs().max().item() <= TOL[dtype]
-    # the log-sum-exp against the rows form (which never tries a tile against an old reference) on the same K/V
+    # the log-sum-exp against the rows form on the same K/V
     gm = torch.cat(c["slots"]).to(torch.int32).to(device)
     gk = torch.empty((gm.numel(), Hkv, d), dtype=dtype, device=device)
     gv = torch.empty_like(gk)
