@@ -1403,8 +1403,8 @@ void pick_qt(const PrefillParams &p, int64_t total_q, hipStream_t stream) {
   // do: head sizes above 128, sliding windows, rows too far apart for 32-bit offsets.
   if constexpr (HDP <= 128) {
     const int force = tuning().prefill_kernel;  // 0: choose here; 1: eight wavefronts; 2 / 3: four wavefronts, 2 / 1 row tiles
-    // the eight-wavefront kernel addresses a tile's 64 rows with 32-bit byte offsets
-    const bool fits = p.k_row < (1 << 23) && p.v_row < (1 << 23);
+    // the eight-wavefront kernel addresses a tile's 64 rows with unsigned 32-bit byte offsets
+    const bool fits = p.k_row >= 0 && p.k_row < (1 << 23) && p.v_row >= 0 && p.v_row < (1 << 23);
     // it knows the causal mask and no mask; other windows go to the four-wavefront kernel
     const bool plain = p.win_left < 0 && p.win_right <= 0;
     if (plain && fits && (force == 0 || force == 1)) {
