@@ -56,8 +56,11 @@
 // -DHIPATTN_PHASE_TRACE=<workgroup id>, lane 0 of every wavefront of that
 // workgroup stores a clock at the phase boundaries of its first 64 tiles (the
 // constant-rate 100 MHz counter, or with -DHIPATTN_PHASE_CYCLES the shader
-// clock); hipattn_debug_phase_trace copies the table out.  Not compiled into
-// normal builds.
+// clock); row 63 of the table takes the workgroup's own marks instead (entry,
+// first period, end of the loop, exit, and the waits of the set-up between
+// them); hipattn_debug_phase_trace copies the table out.  Not compiled into
+// normal builds.  The stamps cost a few hundred cycles per tile: differences
+// between builds mean more than the figures themselves.
 #ifdef HIPATTN_PHASE_TRACE
 __device__ long long g_phase_trace[64 * 8 * 8];
 #ifdef HIPATTN_PHASE_CYCLES
