@@ -139,6 +139,29 @@ def test_strided_qkv_from_a_fused_projection(device):
     assert (got.cpu().double() - fp64(p)).abs().max().item() <= TOL[dtype]
 
 
+def test_random_ragged_cases(device):
+    """Twenty-four seeded draws of dtype, head shape (sizes that fill their MFMA tiles and sizes that do not),
+    batch, new and prior lengths around the tile sizes (1, 63..65, 255..257, 513) and mask, against the fp32
+    oracle: tiles cut by the end of the keys, by the diagonal, by both, and rows with a single key."""
+    rng = np.random.default_rng(11)
+    pick = lambda xs: xs[int(rng.integers(len(xs)))]
+    for case in range(24):
+        dtype = pick([torch.bfloat16, torch.float16])
+        d = pick([32, 40, 64, 72, 80, 96, 104, 128])
+        Hkv = pick([1, 2, 4])
+        Hq = Hkv * pick([1, 2, 4])
+        B = int(rng.integers(1, 4))
+        lens_q = [pick([1, 5, 63, 64, 65, 100, 255, 256, 257, 513]) for _ in range(B)]
+        lens_k = [lq + pick([0, 0, 7, 64, 100, 333, 700]) for lq in lens_q]
+        causal = bool(rng.random() < 0.75)
+        p = general_inputs(100 + case, lens_q, lens_k, Hq, Hkv, d, dtype)
+        got = run(p, device, causal=causal).cpu()
+        want = ref.varlen_attn(p.q.float(), ref.repeat_kv(p.k.float(), Hq // Hkv), ref.repeat_kv(p.v.float(), Hq // Hkv),
+                               p.cu_q, p.cu_k, p.max_q, p.max_k, p.scale, causal)
+        err = (got.float() - want).abs().max().item()
+        assert not torch.isnan(got).any() and err <= TOL[dtype], (case, dtype, d, Hq, Hkv, lens_q, lens_k, causal, err)
+
+
 def bf16_half_ulp(x: torch.Tensor) -> torch.Tensor:
     """Half the spacing of bf16 numbers at |x| (8 significand bits): what storing x as bf16 can cost."""
     return torch.maximum(x.abs(), torch.tensor(2.0 ** -126, dtype=x.dtype)).log2().floor().exp2() * 2.0 ** -8
