@@ -121,6 +121,26 @@ def test_scores_that_drift_along_the_keys(device, dtype, slope):
         assert torch.allclose(lse[i, :, :lq], lse2[i, :, :lq], atol=2e-3, rtol=1e-4)
 
 
+def test_random_ragged_cases(device):
+    """Sixteen seeded draws of dtype, head shape, batch, and new and prior lengths around the tile and block
+    sizes, through the paged cache against the oracle's route."""
+    rng = np.random.default_rng(12)
+    pick = lambda xs: xs[int(rng.integers(len(xs)))]
+    for case in range(16):
+        dtype = pick([torch.bfloat16, torch.float16])
+        d = pick([32, 40, 64, 80, 96, 120, 128])
+        Hkv = pick([1, 2, 4])
+        Hq = Hkv * pick([1, 2, 4])
+        seqs = [(pick([0, 0, 7, 16, 64, 100, 333, 700]), pick([1, 5, 15, 16, 17, 63, 64, 65, 255, 257, 513]))
+                for _ in range(int(rng.integers(1, 4)))]
+        pool = sum((a + b + 15) // 16 for a, b in seqs) + 3
+        c = paged_case(200 + case, seqs, Hq, Hkv, d, dtype, pool)
+        got = run_paged(c, device).cpu()
+        want = oracle(c, Hq, Hkv, d)
+        err = (got.float() - want).abs().max().item()
+        assert not torch.isnan(got).any() and err <= TOL[dtype], (case, dtype, d, Hq, Hkv, seqs, err)
+
+
 def test_agrees_with_gather_then_contiguous_prefill_and_lse(device):
     dtype = torch.bfloat16
     Hq, Hkv, d = 32, 8, 128
