@@ -66,10 +66,12 @@ __device__ long long g_phase_trace[64 * 8 * 8];
 #ifdef HIPATTN_PHASE_CYCLES
 #define wall_clock64 __builtin_readcyclecounter
 #endif
-#define PHASE_STAMP(slot)                                                                                        \
+#define PHASE_STAMP_AT(tile, slot)                                                                               \
   do {                                                                                                           \
-    if (blockIdx.x == HIPATTN_PHASE_TRACE && j < 64 && lane == 0) g_phase_trace[(j * 8 + wave) * 8 + (slot)] = wall_clock64(); \
+    if (blockIdx.x == HIPATTN_PHASE_TRACE && (tile) < 63 && lane == 0)                                           \
+      g_phase_trace[((tile) * 8 + wave) * 8 + (slot)] = wall_clock64();                                         \
   } while (0)
+#define PHASE_STAMP(slot) PHASE_STAMP_AT(j, slot)
 #define PHASE_MARK(slot)                                                                                        \
   do {                                                                                                           \
     if (blockIdx.x == HIPATTN_PHASE_TRACE && (threadIdx.x & 63) == 0) g_phase_trace[(63 * 8 + (threadIdx.x >> 6)) * 8 + (slot)] = wall_clock64(); \
@@ -77,6 +79,9 @@ __device__ long long g_phase_trace[64 * 8 * 8];
 #else
 #define PHASE_STAMP(slot) \
   do {                    \
+  } while (0)
+#define PHASE_STAMP_AT(tile, slot) \
+  do {                             \
   } while (0)
 #define PHASE_MARK(slot) \
   do {                   \
@@ -1170,9 +1175,9 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     auto v_block = [&](int t) {
       if (!skip_tile(t)) qk_softmax(std::false_type{}, t, s_a, s_b, pk);
       if constexpr (DMA) {
-        { const int j = t; PHASE_STAMP(4); }
+        PHASE_STAMP_AT(t, 4);
         if (t + 2 < n_tiles) dma_wait(t + 2, false);
-        { const int j = t; PHASE_STAMP(5); }
+        PHASE_STAMP_AT(t, 5);
         if (t + 3 < n_tiles) dma_tile(t + 3);
       } else {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's pieces of tile t + 2
