@@ -41,11 +41,7 @@
 // error (2^-9 relative in bf16, 2^-12 in fp16); the normaliser is given the
 // same rounding for each half-tile's largest term so that it cancels where it
 // matters, on rows that one key dominates.
-#include <type_traits>
-
-#include "common.h"
-#include "device_types.h"
-#include "workspace.h"
+#include "prefill_common.h"
 
 // The global -> LDS copies below set M0 inside inline asm and say so in their clobber lists, so that the
 // compiler never assumes a value of its own survives them.  M0 is a register the compiler reserves, and
@@ -92,92 +88,7 @@ namespace hipattn {
 
 namespace {
 
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
 constexpr int BN = 64;  // keys per LDS tile
-
-struct PrefillParams {
-  const void *q, *k, *v;
-  void *out;
-  float *lse;  // [batch, Hq, max_q] or null
-  int64_t q_row, q_head, k_row, k_head, v_row, v_head, o_row, o_head;
-  const int32_t *cu_q, *cu_k, *seqused_k;
-  int batch, Hq, Hkv, G, d;
-  int max_q;      // caller's bound on Lq; sizes the grid
-  int lse_pitch;  // elements between (batch, head) rows of lse
-  int n_qblocks;
-  float scale_log2;
-  int causal;  // win_left < 0 && win_right == 0
-  // Query row i (0-based in its sequence) sees key j iff i + off - win_left <= j <= i + off + win_right,
-  // off = Lk - Lq; a negative bound is no bound (flash_attn/softmax.h:142-179, flash_api.cpp:113-120).
-  // Only prefill_varlen_kernel reads these; the eight-wavefront kernel takes causal or unmasked launches.
-  int win_left, win_right;
-  // K/V read straight from the paged cache (prefill_varlen_w8_kernel<..., W8_PAGED or W8_PAGED_DMA>): k and v are
-  // the caches, position p of sequence b lives in block block_tables[b][p / 16] at offset p % 16.
-  const int32_t *block_tables;
-  const int32_t *context_lens;  // keys per sequence
-  int64_t table_stride;
-  int table_cols;
-  int64_t num_blocks;
-  int64_t kc_block, kc_head, vc_block, vc_head;  // cache strides in elements
-  // out holds fp32 instead of the input type: the accumulators divided by the row sums, not rounded again
-  // (for checking the kernel's arithmetic apart from the rounding of its output; o_row / o_head count floats).
-  int out_f32;
-  float rescale_thr;
-  // Eight-wavefront kernel: a workgroup covers 2^wg_heads_log2 query heads of one kv group, 256 >> wg_heads_log2
-  // query rows of each (wavefront w: head w % heads, row group w / heads).
-  int wg_heads_log2;  // a row's reference maximum moves when the row outgrows it by more than this (log2 units)
-};
-
-template <typename T>
-struct Mfma32;
-template <>
-struct Mfma32<half_t> {
-  __device__ static __forceinline__ f32x16_t run(half8_t a, half8_t b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  }
-};
-template <>
-struct Mfma32<bf16_t> {
-  __device__ static __forceinline__ f32x16_t run(bf16x8_t a, bf16x8_t b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-};
-
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-
-// max(a, b, c) in one instruction.  Scores are never NaN here, so the
-// canonicalising copies fmaxf would add to every MFMA result are not needed.
-// Workgroup barrier for LDS hand-offs: waits for this wavefront's LDS
-// operations only.  __syncthreads() also drains the vector-memory counter,
-// which would make every tile wait for the global loads of the tile after next
-// that were just issued.
-// A pointer that is the same in every lane, as the scalar it is: an "s" operand of inline asm is not made one
-// when the compiler holds the value in vector registers.
-template <typename P>
-__device__ __forceinline__ const P *uniform_ptr(const P *ptr) {
-  const uint64_t v = reinterpret_cast<uint64_t>(ptr);
-  return reinterpret_cast<const P *>(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32)) << 32) |
-                                     (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v));
-}
-__device__ __forceinline__ void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-// Maximum of a value and its counterpart in the other half of the wavefront
-// (lane ^ 32), through the gfx950 half-swap instead of an LDS permute.
-__device__ __forceinline__ float max_across_halves(float x) {
-  const unsigned u = bit_cast<unsigned>(x);
-  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return fmaxf(bit_cast<float>((unsigned)r[0]), bit_cast<float>((unsigned)r[1]));
-}
-
-__device__ __forceinline__ float max3(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
 
 // Row strides of the LDS tiles in elements.  K is read as 16 B per lane with
 // 16 consecutive rows per access phase, V as 64 B runs of 4 consecutive rows;
@@ -1561,6 +1472,8 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
   p.win_right = win_right;
   p.out_f32 = out->dtype == HIPATTN_F32 ? 1 : 0;
   p.rescale_thr = (float)tuning().prefill_rescale_log2;
+  const int force = tuning().prefill_kernel;
+  if ((force == 4 || (force == 0 && prefer_prefill_r3(p))) && launch_prefill_r3(p, q->dtype, stream)) return;
   if (q->dtype == HIPATTN_F16) dispatch_hd<half_t>(p, total_q, stream);
   else dispatch_hd<bf16_t>(p, total_q, stream);
 }

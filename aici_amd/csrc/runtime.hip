@@ -78,7 +78,7 @@ const TuningField kTuningFields[] = {
     {"decode_flat", &Tuning::decode_flat, -1, 1},
     {"decode_flat_wgs", &Tuning::decode_flat_wgs, 0, 1 << 16},
     {"decode_part_blocks", &Tuning::decode_part_blocks, 0, 64},
-    {"prefill_kernel", &Tuning::prefill_kernel, 0, 3},
+    {"prefill_kernel", &Tuning::prefill_kernel, 0, 4},
     {"paged_prefill_dma", &Tuning::paged_prefill_dma, -1, 1},
     {"cache_move_lds", &Tuning::cache_move_lds, -1, 1},
     {"prefill_wg_heads", &Tuning::prefill_wg_heads, 0, 8},

@@ -27,7 +27,7 @@ struct Tuning {
   int decode_flat;         // -1: the library chooses; 0 / 1: partitioned / flat-split launch
   int decode_flat_wgs;     // 0: what the device holds at once; else workgroups of the flat launch
   int decode_part_blocks;  // 0: chosen per call; else KV blocks per partition (2..64)
-  int prefill_kernel;      // 0: the library chooses; 1: eight wavefronts; 2 / 3: four wavefronts, 2 / 1 row tiles each
+  int prefill_kernel;      // 0: the library chooses; 1: eight wavefronts; 2 / 3: four wavefronts, 2 / 1 row tiles each; 4: three groups of four
   int paged_prefill_dma;   // -1: the library chooses; 0: staged tiles; 1: block images where possible
   int cache_move_lds;      // -1: the library chooses; 0: never the LDS-transposing kernels
   int prefill_wg_heads;      // eight-wavefront prefill: query heads of one kv group per workgroup, at most (0 and 1: one)

@@ -427,7 +427,8 @@ char *hipattn_shutdown(void);
  * (-1 library's choice, 0 partitioned launch, 1 flat split), decode_flat_wgs
  * (0 = what the device holds at once), decode_part_blocks (0 = chosen per
  * call, else 2..64), prefill_kernel (0 library's choice, 1 eight wavefronts,
- * 2 / 3 four wavefronts with 2 / 1 row tiles), paged_prefill_dma (-1 library's
+ * 2 / 3 four wavefronts with 2 / 1 row tiles, 4 three groups of four
+ * wavefronts), paged_prefill_dma (-1 library's
  * choice, 0 staged tiles), cache_move_lds (-1 library's choice, 0 never the
  * LDS-transposing kernels), prefill_wg_heads (query heads of one kv group per
  * workgroup of the eight-wavefront prefill kernel, at most; 0 and 1: one),

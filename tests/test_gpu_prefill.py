@@ -15,12 +15,13 @@ from tests.common import TOL, kat_inputs, load_kat, round4
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["auto", "eight_wavefronts", "four_wavefronts"])
+@pytest.fixture(autouse=True, params=["auto", "eight_wavefronts", "four_wavefronts", "three_groups"])
 def kernel_choice(request, tuning):
-    """The forward pass has two kernels (256-row workgroups of eight wavefronts for head sizes up to
-    128, 128-row workgroups of four) and picks by launch size; every test runs under the library's
-    own choice and with each one forced (head sizes above 128 always take the second)."""
-    tuning("prefill_kernel", {"auto": 0, "eight_wavefronts": 1, "four_wavefronts": 3}[request.param])
+    """The forward pass has three kernels (256-row workgroups of eight wavefronts and 96- or 384-row
+    workgroups of three groups of four wavefronts for head sizes up to 128, 128-row workgroups of four
+    for the rest) and picks by shape; every test runs under the library's own choice and with each one
+    forced (what a forced kernel does not cover falls through to the one that does)."""
+    tuning("prefill_kernel", {"auto": 0, "eight_wavefronts": 1, "four_wavefronts": 3, "three_groups": 4}[request.param])
     return request.param
 
 
