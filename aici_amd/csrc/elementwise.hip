@@ -333,13 +333,20 @@ __global__ __launch_bounds__(1024) void bias_argmax_kernel(const T *__restrict__
 // among equals.  A slice's winner is one 64-bit key -- the value's bits made
 // monotonic above, the complement of the id below -- so the best slice of a
 // row is a device-wide atomic maximum; the workgroup that counts in last reads
-// it, writes the row's result and puts key and counter back to zero for the
-// next call (row_state: {key, counter} per row, zero before the first call).
+// it and writes the row's result (row_state: {key, counter} per row, cleared by
+// a small fill kernel in front of every launch, so that whatever an overlapping
+// or interrupted call left there cannot reach a later one).
 struct ArgmaxRowState {
   unsigned long long key;
   unsigned int arrived;
   unsigned int pad;
 };
+
+// (a kernel, not hipMemsetAsync: the call may be recorded into a graph)
+__global__ void argmax_state_clear_kernel(ArgmaxRowState *__restrict__ st, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) st[i] = ArgmaxRowState{0ull, 0u, 0u};
+}
 
 __device__ __forceinline__ unsigned long long argmax_key(float v, int idx) {
   const unsigned int b = __float_as_uint(v);
@@ -430,7 +437,6 @@ __global__ __launch_bounds__(256) void bias_argmax_slice_kernel(const T *__restr
       if (token == 0x7fffffff) token = 0;  // every token disallowed: torch's argmax of equal -inf is 0
       out_tokens[seq] = token;
       if (out_logits) out_logits[seq] = __uint_as_float((mono & 0x80000000u) ? (mono & 0x7fffffffu) : ~mono);
-      __hip_atomic_exchange(&st->arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 }
@@ -688,9 +694,11 @@ void bias_argmax_impl(const hipattn_tensor *logits, const hipattn_tensor *bias, 
     if (chunks < 1) chunks = 1;
     const int per_slice = (int)((((V + chunks - 1) / chunks) + 7) / 8 * 8);
     chunks = (V + per_slice - 1) / per_slice;
-    // Zero when allocated, and every call leaves it zero.
+    // The row states are cleared on the stream in front of every launch: a call never depends on what the
+    // one before it (or a replay of a captured graph overlapping it on another stream) left behind.
     ArgmaxRowState *st =
         static_cast<ArgmaxRowState *>(library_workspace(WS_BIAS_ARGMAX, (size_t)S * sizeof(ArgmaxRowState), stream));
+    argmax_state_clear_kernel<<<dim3((unsigned)((S + 255) / 256)), 256, 0, stream>>>(st, (int)S);
     int32_t *ot = static_cast<int32_t *>(out_tokens->data);
     const dim3 grid((unsigned)chunks, (unsigned)S);
 #define HA_BAW(TT)                                                                                               \

@@ -28,6 +28,7 @@ namespace {
 thread_local hipStream_t tl_current_stream = nullptr;
 std::mutex g_mutex;
 int64_t g_peak[64];
+int64_t g_lib_allocated[64], g_lib_freed[64];  // bytes of device memory this library itself has allocated / released
 constexpr int kMaxDevices = 64;
 
 // Library-owned scratch: one buffer per (op, device, stream).  `retired` holds the buffers that a
@@ -102,7 +103,12 @@ void *library_workspace(WorkspaceUser user, size_t bytes, hipStream_t stream) {
   if (ws.bytes >= bytes && ws.ptr != nullptr) return ws.ptr;
   // Allocating is not something a capture can record, and the graph would keep the old pointer.
   hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) (void)hipGetLastError();
+  const hipError_t asked = hipStreamIsCapturing(stream, &capturing);
+  if (asked != hipSuccess) {
+    (void)hipGetLastError();
+    fail("hipStreamIsCapturing failed (%s): cannot tell whether the library's scratch buffer may grow on this stream",
+         hipGetErrorString(asked));
+  }
   HA_CHECK(capturing == hipStreamCaptureStatusNone,
            "the library's scratch buffer for this stream must grow to %zu bytes, which cannot happen while the stream is "
            "being captured: run the call once outside the capture first, or use the entry point that takes a workspace",
@@ -119,6 +125,7 @@ void *library_workspace(WorkspaceUser user, size_t bytes, hipStream_t stream) {
     fail("clearing a new scratch buffer failed: %s", hipGetErrorString(e));
   }
   if (ws.ptr != nullptr) g_retired.emplace_back(dev, ws.ptr);
+  g_lib_allocated[dev] += (int64_t)want;
   ws.ptr = fresh;
   ws.bytes = want;
   return ws.ptr;
@@ -211,6 +218,7 @@ extern "C" char *hipattn_shutdown(void) {
       if (kv.second.ptr) all.emplace_back(kv.first.device, kv.second.ptr);
     g_retired.clear();
     g_scratch.clear();
+    for (int dv = 0; dv < kMaxDevices; dv++) g_lib_freed[dv] = g_lib_allocated[dv];
     int synced = -1;
     for (auto &dp : all) {
       HA_HIP(hipSetDevice(dp.first));
@@ -281,8 +289,8 @@ extern "C" char *hipattn_get_stats_allocated_bytes(int device, hipattn_mem_stats
     if (used > g_peak[device]) g_peak[device] = used;
     outp->current = used;
     outp->peak = g_peak[device];
-    outp->allocated = 0;
-    outp->freed = 0;
+    outp->allocated = g_lib_allocated[device];
+    outp->freed = g_lib_freed[device];
   });
 }
 

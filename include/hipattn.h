@@ -311,7 +311,14 @@ char *hipattn_gelu_fast(hipattn_tensor *out, const hipattn_tensor *input,
  *         8*mask_bytes are disallowed.
  * bias_rows int32 [S] or NULL selects the row for each sequence (identity when
  * NULL).  out_tokens int32 [S]; out_logits f32 [S] or NULL receives the
- * winning biased logit.  Ties resolve to the lowest token id. */
+ * winning biased logit.  Ties resolve to the lowest token id.
+ * For large vocabularies the call keeps a few bytes of state per row in a
+ * library-owned buffer that belongs to the stream it runs on (cleared by the
+ * call itself, so no call depends on an earlier one).  Calls that share that
+ * buffer must not overlap: a graph captured from this call replays onto the
+ * buffer of the stream it was captured on, so two replays of such graphs on
+ * different streams at once, or a replay beside eager calls on the capture
+ * stream, give wrong tokens for the overlapping calls (never for later ones). */
 char *hipattn_bias_argmax(const hipattn_tensor *logits,
                           const hipattn_tensor *bias,
                           const hipattn_tensor *mask,
@@ -370,7 +377,9 @@ typedef struct hipattn_device_props {
  * cuda_get_stats_allocated_bytes_C / cuda_get_device_properties_C
  * (cuda.cpp:34-60).  Without a caching allocator the figures come from
  * hipMemGetInfo: current = total - free on the device, peak = the largest
- * `current` seen by any stats call since the last reset. */
+ * `current` seen by any stats call since the last reset; allocated / freed =
+ * the bytes of scratch memory this library itself has allocated on the device
+ * and released again (hipattn_shutdown) since it was loaded. */
 char *hipattn_reset_peak_memory_stats(int device);
 char *hipattn_empty_cache(void); /* nothing to release: no caching allocator; see hipattn_shutdown */
 char *hipattn_get_stats_allocated_bytes(int device, hipattn_mem_stats *outp);

@@ -221,6 +221,30 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
     return out
 
 
+def paged_attention_fp64(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, num_kv_heads: int,
+                         scale: float, block_tables: torch.Tensor, context_lens: torch.Tensor,
+                         block_size: int) -> torch.Tensor:
+    """The same rows as paged_attention (Lq = 1 varlen attention over the gathered context, refkernels.rs:59-148
+    behind batch_info.rs:209-220), stated once more in float64 with whole-block indexing instead of the slot
+    loop, so that every row of a full-size step can be checked in seconds.  Rounds nothing: the result is the
+    exact softmax(K q * scale) V of the given numbers, returned as float64 [S, Hq, d]."""
+    S, Hq, d = query.shape
+    g = Hq // num_kv_heads
+    out = torch.zeros((S, Hq, d), dtype=torch.float64)
+    for s in range(S):
+        ctx = int(context_lens[s])
+        if ctx == 0:
+            continue
+        blocks = block_tables[s, :(ctx + block_size - 1) // block_size].long()
+        # key cache [nb, Hkv, d/x, bs, x] -> [tokens, Hkv, d]; value cache [nb, Hkv, d, bs] -> [tokens, Hkv, d]
+        kk = key_cache[blocks].permute(0, 3, 1, 2, 4).reshape(-1, num_kv_heads, d)[:ctx].double()
+        vv = value_cache[blocks].permute(0, 3, 1, 2).reshape(-1, num_kv_heads, d)[:ctx].double()
+        q = query[s].double().reshape(num_kv_heads, g, d)
+        p = torch.softmax(torch.einsum("kgd,tkd->kgt", q, kk) * scale, dim=-1)
+        out[s] = torch.einsum("kgt,tkd->kgd", p, vv).reshape(Hq, d)
+    return out
+
+
 # ----------------------------------------------------------------------------- rotary / norm / activations
 
 def rotary_table(rotary_dim: int, rope_theta: float, max_len: int, dtype: torch.dtype) -> torch.Tensor:

@@ -130,8 +130,10 @@ def test_config4_full_size_sampled(device, layout, paged_prefill):
     tokens + 120 decode rows with contexts U[1k, 8k], 32 MHA heads, d 80, fp16 -- with contiguous
     q, k, v and with q, k, v as views of one fused [T, 3, H, d] projection (token stride 3*H*d, what
     Phi's layer passes, phi.rs:131-145), the latter also with the multi-token rows reading the cache
-    through block tables.  The oracle runs on the 4 chunks' last rows and a sample of decode rows
-    (every row is independent)."""
+    through block tables.  The check (a float64 softmax over the row's gathered context; every row is
+    independent) runs on 72 rows: of every chunk its first and last rows and the rows either side of the
+    32-, 64-, 96- and 256-row boundaries that the kernels' row blocks and wavefronts cut at, and 24 decode
+    rows, the shortest and the longest context among them."""
     rng = np.random.default_rng(4)
     g = torch.Generator().manual_seed(4)
     Hq = Hkv = 32
@@ -169,8 +171,10 @@ def test_config4_full_size_sampled(device, layout, paged_prefill):
     assert not torch.isnan(y.float()).any()
     kc, vc = kd.cpu(), vd.cpu()  # after the step: holds the new tokens too
     worst = 0.0
-    samples = [(512 * (i + 1) - 1, None) for i in range(4)] + [(0, None), (1500, None)]
-    samples += [(2048 + int(r), int(r)) for r in rng.choice(120, size=10, replace=False)]
+    samples = [(512 * i + r, None) for i in range(4) for r in (0, 1, 31, 32, 63, 64, 95, 96, 255, 256, 300, 511)]
+    dec_rows = {int(np.argmin(ctxs)), int(np.argmax(ctxs)), *(int(r) for r in rng.choice(120, size=22, replace=False))}
+    samples += [(2048 + r, r) for r in sorted(dec_rows)]
+    assert len(samples) >= 64
     for row, paged_row in samples:
         if paged_row is None:
             e = row // 512

@@ -176,3 +176,66 @@ def test_full_width_layer_lm_head_and_mask_at_llama3_8b_shape(device):
     for sid, t in zip([1, 2, 3, 4, 5], toks.tolist()):
         sides.append(sid, int(t))
     run([3, 1, 5, 2, 4])
+
+
+def test_32_layer_step_at_llama3_8b_shape_properties(device):
+    """The full-model configuration's step at its own size -- 32 layers, hidden 4096, FFN 14336, vocabulary
+    128256, 128 sequences decoding one token over contexts U[1024, 16384] (seed 5), bf16, 5 % allow-mask --
+    with one KV cache shared by the layers (each layer reads and writes the same 4.6 GB).  No CPU side can
+    follow 32 layers at this width in a test's time (one layer and the lm_head against the CPU build is the
+    test above), so this one checks what does not need it: every constrained token is an allowed one; the
+    fused call sequence (rotary + cache scatter in one launch, q / k / v as views of the projection) gives
+    the tokens of the reference's call sequence; the step is repeatable; and a HIP graph of it replays to
+    the same tokens three times with eager work in between."""
+    cfg = llama.LlamaConfig.llama3_8b()
+    assert (cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size) == (32, 4096, 14336, 128256)
+    rng = np.random.default_rng(5)
+    S = 128
+    ctx = rng.integers(1024, 16384 + 1, size=S)
+    pool = int(((ctx + 15) // 16).sum()) + 64
+    alloc = paged.BlockAllocator(16, pool)
+    builder = paged.BatchInfoBuilder(16, cfg.max_position_embeddings, 1)
+    for sid, n in enumerate(ctx.tolist(), start=1):
+        alloc.alloc_seq(sid, n)
+        builder.sched_out(alloc, sid, rng.integers(0, cfg.vocab_size, size=n).astype(np.int32), n - 1)
+    bi = builder.finish().to(device)
+    model = llama.Llama(cfg, llama.random_weights(cfg, 5, device=device), device)
+    g = torch.Generator(device=device).manual_seed(5)
+    kc, vc = paged.alloc_gpu_cache_layer(pool, cfg.num_key_value_heads, cfg.head_dim, 16, cfg.dtype, device)
+    kc.normal_(generator=g)
+    vc.normal_(generator=g)
+    caches = [(kc, vc)] * cfg.num_hidden_layers
+    allowed = W.allow_mask(5, S, cfg.vocab_size)
+    assert 0.04 < allowed.mean() < 0.06
+    masks = torch.from_numpy(np.stack([oaici.pack_allowed(a) for a in allowed])).to(device)
+
+    def step(fused=True):
+        return llama.aici_greedy(model.forward(bi, caches, fused=fused), masks)
+
+    # Every layer writes this step's keys and values into the shared cache at the same slots; after the first
+    # step the cache holds the last layer's, and from then on a step reads and writes the same values: the
+    # second step is the reference point.
+    step()
+    toks = step()
+    torch.cuda.synchronize()
+    t = toks.cpu().long()
+    assert t.shape == (S,) and bool(torch.from_numpy(allowed)[torch.arange(S), t].all())
+    assert len(set(t.tolist())) > S // 2          # not one token for everybody
+    assert torch.equal(step(), toks)              # repeatable
+    assert torch.equal(step(False), toks)         # the reference's call sequence
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                    # sizes this stream's scratch buffers outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        toks_graph = step()
+    for _ in range(3):
+        toks_graph.fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(toks_graph, toks)
+        assert torch.equal(step(), toks)          # eager work between the replays

@@ -176,16 +176,20 @@ def test_invariant_under_block_permutation_and_equals_prefill_last_row(device):
 
 
 def test_config2_full_size(device):
-    """The benchmark's decode configuration at full size: every sequence against the oracle."""
+    """The benchmark's decode configuration at full size: every one of the 64 sequences against the float64
+    statement of the oracle, and every third one against the slot-by-slot oracle itself."""
     c = W.config2()
     assert c.q.shape == (64, 32, 128) and c.key_cache.shape == (20000, 8, 16, 16, 8)
     got = run_v1(c, device)
     assert not torch.isnan(got).any()
-    rows = list(range(0, 64, 3))  # 22 of the 64 sequences through the (slow) oracle
     if "config2" not in _ORACLE_CACHE:
-        _ORACLE_CACHE["config2"] = oracle(c, rows=rows)
-    want = _ORACLE_CACHE["config2"]
+        rows = list(range(0, 64, 3))
+        _ORACLE_CACHE["config2"] = (rows, oracle(c, rows=rows),
+                                    ref.paged_attention_fp64(c.q, c.key_cache, c.value_cache, c.num_kv_heads, c.scale,
+                                                             c.block_tables, c.context_lens, 16))
+    rows, want, want64 = _ORACLE_CACHE["config2"]
     assert (got[rows].float() - want).abs().max().item() <= TOL[torch.bfloat16]
+    assert (got.double() - want64).abs().max().item() <= TOL[torch.bfloat16]
     # size-independent property on all 64: attention output is a convex combination of the
     # context's V rows, so each coordinate lies within the range of that kv head's values
     assert got.float().abs().max().item() <= c.value_cache.float().abs().max().item()
@@ -276,6 +280,11 @@ def test_other_block_sizes_edges_alibi_and_stale_slots(device, dtype, bs):
                          c.max_ctx, alibi.to(device))
     assert not torch.isnan(out).any()
     assert torch.all(out[0] == 0)   # no context: a zero row, as the oracle gives
+    # one token of context: its value, exactly -- the normaliser is 1 / sum as in rLLM's CPU reference kernels
+    # (refkernels.rs:59-148), not the CUDA kernel's 1 / (sum + 1e-6) (attention_kernels.cu:262), which would give
+    # v / (1 + 1e-6) and shows in float32
+    one = c.value_cache[int(tables[1, 0]), :, :, 0].repeat_interleave(4, dim=0)   # [Hq, d]: 8 q heads on 2 kv heads
+    assert torch.equal(out[1].cpu(), one.to(dtype))
     tol = 5e-5 if dtype == torch.float32 else TOL[dtype]
     assert (out.cpu().float() - want).abs().max().item() <= tol
 
@@ -372,9 +381,10 @@ def test_context_lengths_above_the_stated_maximum_are_cut_there(device, dtype, b
 def test_config5_decode_shape(device):
     """The decode attention of the full-model configuration at its own shape: 128 sequences with contexts
     U[1024, 16384] (seed 5), 32 q / 8 kv heads, d 128, bf16 -- 1.1 M context tokens, 4.6 GB of K/V in a
-    70k-block pool.  The cache is filled on the GPU (seeded); 18 sequences, the shortest and the longest
-    among them, are checked against the oracle on their own blocks brought to the CPU, all 128 by the range
-    property (an attention output is a convex combination of its context's V rows)."""
+    70k-block pool.  The cache is filled on the GPU (seeded); every sequence is checked against the float64
+    statement of the oracle on its own blocks brought to the CPU, 18 of them -- the shortest and the longest
+    among them -- against the slot-by-slot oracle as well, and all by the range property (an attention
+    output is a convex combination of its context's V rows)."""
     rng = np.random.default_rng(5)
     S = 128
     ctx = rng.integers(1024, 16384 + 1, size=S)
@@ -396,6 +406,16 @@ def test_config5_decode_shape(device):
             kc, vc = c.key_cache[blocks].cpu(), c.value_cache[blocks].cpu()   # this sequence's blocks, renumbered 0..n-1
             want.append(ref.paged_attention(c.q[s:s + 1].cpu().float(), kc.float(), vc.float(), 8, c.scale,
                                             torch.arange(n, dtype=torch.int32)[None], c.context_lens[s:s + 1].cpu(), 16)[0])
-        _ORACLE_CACHE["config5"] = torch.stack(want)
-    err = (out[rows].cpu().float() - _ORACLE_CACHE["config5"]).abs().max().item()
+        want64 = []
+        for s in range(S):
+            n = (int(ctx[s]) + 15) // 16
+            blocks = c.block_tables[s, :n].long()
+            want64.append(ref.paged_attention_fp64(c.q[s:s + 1].cpu(), c.key_cache[blocks].cpu(), c.value_cache[blocks].cpu(),
+                                                   8, c.scale, torch.arange(n, dtype=torch.int32)[None],
+                                                   c.context_lens[s:s + 1].cpu(), 16)[0])
+        _ORACLE_CACHE["config5"] = (torch.stack(want), torch.stack(want64))
+    want, want64 = _ORACLE_CACHE["config5"]
+    err = (out[rows].cpu().float() - want).abs().max().item()
     assert err <= TOL[torch.bfloat16], err
+    err64 = (out.cpu().double() - want64).abs().max().item()
+    assert err64 <= TOL[torch.bfloat16], err64

@@ -165,11 +165,11 @@ def test_bias_argmax_bias_rows_and_packed_mask(device, dtype):
 
 
 def test_bias_argmax_wide_rows_call_after_call(device):
-    """Long 16-bit rows are cut into slices whose winners meet in a per-row key and counter kept between calls:
-    call after call with changing row counts, negative and infinite winners, and the winning value itself."""
+    """Long 16-bit rows are cut into slices whose winners meet in a per-row key and counter in a buffer the
+    library keeps per stream and clears in front of every launch: call after call with changing row counts,
+    vocabularies and slice counts, negative and infinite winners, and the winning value itself."""
     g = torch.Generator().manual_seed(11)
-    V = 65536
-    for S in (128, 5, 64, 1):
+    for S, V in ((128, 65536), (5, 65536), (64, 131072), (1, 65536), (200, 16384), (3, 131072)):
         logits = (torch.randn((S, V), generator=g) - 6.0).to(torch.bfloat16)      # every value negative
         logits[0, 4242] = float("-inf")
         allowed = torch.rand((S, V), generator=g) < 0.03
@@ -183,6 +183,7 @@ def test_bias_argmax_wide_rows_call_after_call(device):
             tok, best = K.bias_argmax(logits.to(device), mask=packed.to(device), return_logits=True)
             assert torch.equal(tok.cpu().long(), want)
             assert torch.equal(best.cpu(), masked[torch.arange(S), want])
+    V = 65536
     pos_inf = torch.zeros((2, V), dtype=torch.float16, device=device)
     pos_inf[1, 40000] = float("inf")
     tok, best = K.bias_argmax(pos_inf, mask=torch.full((2, V // 8), 255, dtype=torch.uint8, device=device),

@@ -186,6 +186,25 @@ def test_paged_attention_equals_dense_softmax_over_gathered_context():
             assert (out[s, h].double() - p @ V).abs().max().item() < 1e-5
 
 
+def test_paged_attention_fp64_statement_agrees_with_the_slot_by_slot_one():
+    """The float64 whole-block statement used for full-size steps against the slot-by-slot oracle (itself
+    pinned above by a per-head dense softmax), over ragged contexts including 0, 1 and block edges."""
+    for seed in (1, 2, 3):
+        q, kc, vc, tables, ctx = _paged_setup(seed)
+        Hkv, bs = kc.shape[1], kc.shape[3]
+        a = ref.paged_attention(q, kc, vc, Hkv, 0.25, tables, ctx, bs)
+        b = ref.paged_attention_fp64(q, kc, vc, Hkv, 0.25, tables, ctx, bs)
+        assert b.dtype == torch.float64 and (a.double() - b).abs().max().item() < 1e-5
+    # a context of one token is that token's value, exactly
+    q, kc, vc, tables, ctx = _paged_setup(4)
+    ctx[:] = 1
+    Hkv, bs = kc.shape[1], kc.shape[3]
+    b = ref.paged_attention_fp64(q, kc, vc, Hkv, 0.25, tables, ctx, bs)
+    for s in range(q.shape[0]):
+        for h in range(q.shape[1]):
+            assert torch.equal(b[s, h], vc[int(tables[s, 0]), h // (q.shape[1] // Hkv), :, 0].double())
+
+
 def test_paged_attention_invariant_under_block_permutation_and_equals_prefill_last_row():
     q, kc, vc, tables, ctx = _paged_setup(2)
     Hkv, bs = kc.shape[1], kc.shape[3]

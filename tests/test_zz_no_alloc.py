@@ -46,3 +46,46 @@ def test_static_scratch_entry_refuses_what_does_not_fit(device, tuning):
     with pytest.raises(HipAttnError, match="more than the 16777216 bytes of the built-in array"):
         K.paged_attention_v1_static(out, d.q, d.key_cache, d.value_cache, 8, c.scale, d.block_tables, d.context_lens,
                                     16, c.max_ctx)
+
+
+@pytest.mark.filterwarnings("ignore:The CUDA Graph is empty")   # the refused capture records nothing, as it should
+def test_capture_on_a_cold_stream(device, tuning):
+    """What the entry point is for: on a stream the library has never seen, under graph capture, v1 has no
+    scratch buffer and may not allocate one -- it must say so -- while the static-array form and the
+    caller-workspace form record and replay, and give v1's bits."""
+    tuning("decode_flat", 1)
+    K.init()
+    c = W.decode_inputs(64, 24, 600, 3000, 32, 8, 128, torch.bfloat16, 24 * 200)
+    d = c.to(device)
+    args = (d.q, d.key_cache, d.value_cache, c.num_kv_heads, c.scale, d.block_tables, d.context_lens, 16, c.max_ctx)
+    want = torch.empty_like(d.q)
+    K.paged_attention_v1(want, *args)                    # eager, on the default stream: kernels loaded, attributes set
+    warm = torch.empty_like(d.q)
+    K.paged_attention_v1_static(warm, *args)
+    ws = torch.empty(K.paged_attention_workspace_size(24, 32, 8, 128, 16, c.max_ctx, torch.bfloat16), dtype=torch.uint8,
+                     device=device)
+    torch.cuda.synchronize()
+    before = K.cuda_get_stats_allocated_bytes(0).allocated
+
+    refused = torch.cuda.Stream()
+    graph0 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph0, stream=refused):
+        with pytest.raises(HipAttnError, match="cannot happen while the stream is being captured"):
+            K.paged_attention_v1(torch.empty_like(d.q), *args)
+
+    cold = torch.cuda.Stream()
+    got_static = torch.full_like(d.q, float("nan"))
+    got_ws = torch.full_like(d.q, float("nan"))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=cold):
+        K.paged_attention_v1_static(got_static, *args)
+        K.paged_attention_v1_ws(got_ws, *args, ws)
+    for _ in range(3):
+        got_static.fill_(float("nan"))
+        got_ws.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got_static, want) and torch.equal(got_ws, want)
+    # nothing was allocated by the library on the way (its own counter of device allocations)
+    assert K.cuda_get_stats_allocated_bytes(0).allocated == before
