@@ -97,7 +97,6 @@ _ERR_FUNCS = {
     "hipattn_gelu_fast": [TP, TP, c_void_p],
     "hipattn_bias_argmax": [TP, TP, TP, TP, TP, TP, c_void_p],
     "hipattn_bias_sample": [TP, TP, TP, TP, TP, TP, TP, TP, c_void_p],
-    "hipattn_stream_probe": [c_int, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p],
     "hipattn_reset_peak_memory_stats": [c_int],
     "hipattn_empty_cache": [],
     "hipattn_get_stats_allocated_bytes": [c_int, POINTER(MemStats)],

@@ -1,4 +1,5 @@
-"""Builds libhipattn.so (the HIP kernels + C ABI) for gfx950 with hipcc.
+"""Builds libhipattn.so (the HIP kernels + C ABI) and libmembench.so (the benchmark's memory-system
+yardsticks, csrc/bench/) for gfx950 with hipcc.
 
     python -m aici_amd.build [--force] [-j N]
 
@@ -21,6 +22,8 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 OBJ = CSRC / "build"
 LIB = PKG / "libhipattn.so"
+BENCH_SRC = CSRC / "bench" / "membench.hip"
+BENCH_LIB = PKG / "libmembench.so"
 
 # -packed-fp32-ops: keep hipcc from forming packed FP32 instructions; the
 # host pass does not know the feature and says so, which is harmless.
@@ -71,6 +74,13 @@ def build(force: bool = False, jobs: int | None = None, verbose: bool = True) ->
             raise RuntimeError(f"link failed:\n{r.stdout}{r.stderr}")
         if verbose:
             print(f"[build] linked {LIB}", flush=True)
+    if force or not BENCH_LIB.exists() or BENCH_LIB.stat().st_mtime < BENCH_SRC.stat().st_mtime:
+        r = subprocess.run(["hipcc", "-shared", "-fPIC", "-O3", "-std=c++17", "--offload-arch=gfx950", str(BENCH_SRC),
+                            "-o", str(BENCH_LIB)], capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {BENCH_SRC.name}:\n{r.stdout}{r.stderr}")
+        if verbose:
+            print(f"[build] linked {BENCH_LIB}", flush=True)
     return LIB
 
 

@@ -1,0 +1,78 @@
+// Memory-system yardsticks for the benchmark: what this device delivers for a plain read, a copy, a fill and
+// a read of shuffled fixed-size chunks -- the figures the decode kernels' bandwidth is held against.  Built into
+// a library of its own (libmembench.so); nothing in the attention library links or calls it.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <algorithm>
+
+namespace {
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Reads `n` 16-byte words once; the xor is stored only if it hits a value it cannot have by chance, so the
+// loads stay and no traffic is written.
+__global__ __launch_bounds__(256) void read_kernel(const u32x4 *__restrict__ src, unsigned int *sink, int64_t n) {
+  unsigned int acc = 0;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const u32x4 v = src[i];
+    acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
+  }
+  if (acc == 0x9e3779b9u && sink) sink[0] = acc;
+}
+__global__ __launch_bounds__(256) void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, int64_t n) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+__global__ __launch_bounds__(256) void fill_kernel(u32x4 *__restrict__ dst, int64_t n) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = u32x4{1u, 2u, 3u, 4u};
+}
+// One workgroup per entry of `chunks`: reads the chunk with that number, `words` 16-byte words long (256 for
+// the 4 KiB in which the paged caches are read: one block of one kv head at head size 128, 16-bit).
+__global__ __launch_bounds__(256) void read_chunks_kernel(const u32x4 *__restrict__ src, const int32_t *__restrict__ chunks,
+                                                           unsigned int *sink, int64_t n_chunks, int words) {
+  unsigned int acc = 0;
+  for (int64_t k = blockIdx.x; k < n_chunks; k += gridDim.x) {
+    const u32x4 *c = src + (int64_t)chunks[k] * words;
+    for (int i = threadIdx.x; i < words; i += 256) {
+      const u32x4 v = c[i];
+      acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
+    }
+  }
+  if (acc == 0x9e3779b9u && sink) sink[0] = acc;
+}
+}  // namespace
+
+// mode 0 reads src once (dst may be null), 1 copies src to dst, 2 fills dst, 3 reads the chunks of src that
+// chunks[0..n_chunks) number (each 0 <= chunks[k] < bytes / chunk_bytes; chunk_bytes a multiple of 4096).
+// Returns 0, a hipError_t, or -1 for bad arguments.
+extern "C" int membench_probe(int mode, void *dst, const void *src, int64_t bytes, const int32_t *chunks, int64_t n_chunks,
+                              int chunk_bytes, void *stream_arg) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_arg);
+  if (bytes < 0 || bytes % 16 != 0) return -1;
+  const int64_t n = bytes / 16;
+  if (n == 0) return 0;
+  const unsigned grid = (unsigned)std::min<int64_t>((n + 255) / 256, 65536);
+  switch (mode) {
+    case 0:
+      if (!src) return -1;
+      read_kernel<<<grid, 256, 0, stream>>>(static_cast<const u32x4 *>(src), static_cast<unsigned int *>(dst), n);
+      break;
+    case 1:
+      if (!src || !dst) return -1;
+      copy_kernel<<<grid, 256, 0, stream>>>(static_cast<const u32x4 *>(src), static_cast<u32x4 *>(dst), n);
+      break;
+    case 2:
+      if (!dst) return -1;
+      fill_kernel<<<grid, 256, 0, stream>>>(static_cast<u32x4 *>(dst), n);
+      break;
+    case 3: {
+      if (!src || !chunks || n_chunks <= 0 || chunk_bytes <= 0 || chunk_bytes % 4096 != 0 || bytes % chunk_bytes != 0) return -1;
+      const unsigned g = (unsigned)std::min<int64_t>(n_chunks, 16384);
+      read_chunks_kernel<<<g, 256, 0, stream>>>(static_cast<const u32x4 *>(src), chunks, static_cast<unsigned int *>(dst), n_chunks,
+                                                chunk_bytes / 16);
+      break;
+    }
+    default: return -1;
+  }
+  return (int)hipGetLastError();
+}

@@ -135,75 +135,6 @@ void *library_workspace(WorkspaceUser user, size_t bytes, hipStream_t stream) {
 
 using namespace hipattn;
 
-// ---- memory-system yardsticks (a measurement aid; nothing in the attention path calls them) ----
-namespace {
-typedef unsigned int probe_u32x4 __attribute__((ext_vector_type(4)));
-
-// Reads `n` 16-byte words once; the xor is stored only if it hits a value it cannot have by chance, so
-// the loads stay and no traffic is written.
-__global__ __launch_bounds__(256) void probe_read_kernel(const probe_u32x4 *__restrict__ src, unsigned int *sink, int64_t n) {
-  unsigned int acc = 0;
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
-    const probe_u32x4 v = src[i];
-    acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
-  }
-  if (acc == 0x9e3779b9u && sink) sink[0] = acc;
-}
-__global__ __launch_bounds__(256) void probe_copy_kernel(const probe_u32x4 *__restrict__ src, probe_u32x4 *__restrict__ dst, int64_t n) {
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) dst[i] = src[i];
-}
-__global__ __launch_bounds__(256) void probe_fill_kernel(probe_u32x4 *__restrict__ dst, int64_t n) {
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
-    dst[i] = probe_u32x4{1u, 2u, 3u, 4u};
-}
-// One workgroup per entry of `chunks`: reads the 4 KiB chunk with that number (256 lanes x 16 bytes) --
-// the granule in which the paged caches are read (one block of one kv head at head size 128, 16-bit).
-__global__ __launch_bounds__(256) void probe_read_chunks_kernel(const probe_u32x4 *__restrict__ src, const int32_t *__restrict__ chunks,
-                                                                 unsigned int *sink, int64_t n_chunks) {
-  unsigned int acc = 0;
-  for (int64_t k = blockIdx.x; k < n_chunks; k += gridDim.x) {
-    const probe_u32x4 v = src[(int64_t)chunks[k] * 256 + threadIdx.x];
-    acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
-  }
-  if (acc == 0x9e3779b9u && sink) sink[0] = acc;
-}
-}  // namespace
-
-extern "C" char *hipattn_stream_probe(int mode, void *dst, const void *src, int64_t bytes, const int32_t *chunks,
-                                      int64_t n_chunks, void *stream_arg) {
-  HA_PROTECT({
-    hipStream_t stream = resolve_stream(stream_arg);
-    HA_CHECK(bytes >= 0 && bytes % 16 == 0, "stream_probe: bytes must be a non-negative multiple of 16");
-    const int64_t n = bytes / 16;
-    if (n == 0) return nullptr;
-    const unsigned grid = (unsigned)std::min<int64_t>((n + 255) / 256, 65536);
-    switch (mode) {
-      case 0:
-        HA_CHECK(src != nullptr, "stream_probe: src is NULL");
-        probe_read_kernel<<<grid, 256, 0, stream>>>(static_cast<const probe_u32x4 *>(src), static_cast<unsigned int *>(dst), n);
-        break;
-      case 1:
-        HA_CHECK(src != nullptr && dst != nullptr, "stream_probe: src or dst is NULL");
-        probe_copy_kernel<<<grid, 256, 0, stream>>>(static_cast<const probe_u32x4 *>(src), static_cast<probe_u32x4 *>(dst), n);
-        break;
-      case 2:
-        HA_CHECK(dst != nullptr, "stream_probe: dst is NULL");
-        probe_fill_kernel<<<grid, 256, 0, stream>>>(static_cast<probe_u32x4 *>(dst), n);
-        break;
-      case 3: {
-        HA_CHECK(src != nullptr && chunks != nullptr && n_chunks > 0, "stream_probe: src, chunks and n_chunks are needed");
-        // the caller guarantees 0 <= chunks[k] < bytes / 4096
-        HA_CHECK(bytes % 4096 == 0, "stream_probe: bytes must be a multiple of 4096 for chunked reads");
-        const unsigned g = (unsigned)std::min<int64_t>(n_chunks, 16384);
-        probe_read_chunks_kernel<<<g, 256, 0, stream>>>(static_cast<const probe_u32x4 *>(src), chunks, static_cast<unsigned int *>(dst), n_chunks);
-        break;
-      }
-      default: fail("stream_probe: mode %d is not one of 0 (read), 1 (copy), 2 (fill), 3 (read 4 KiB chunks)", mode);
-    }
-    check_launch("stream_probe");
-  });
-}
-
 extern "C" void hipattn_free_error(char *msg) { free(msg); }
 
 extern "C" const char *hipattn_version(void) { return "0.1.0"; }

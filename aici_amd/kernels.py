@@ -285,18 +285,6 @@ def bias_sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Te
     return tokens
 
 
-def stream_probe(mode: str, dst: Optional[torch.Tensor], src: Optional[torch.Tensor],
-                 chunks: Optional[torch.Tensor] = None) -> None:
-    """One launch of the library's memory-system yardstick: "read" src once, "copy" src to dst, "fill"
-    dst, or "read_chunks": the 4 KiB chunks of src that the int32 tensor `chunks` numbers."""
-    modes = {"read": 0, "copy": 1, "fill": 2, "read_chunks": 3}
-    t = src if src is not None else dst
-    nbytes = t.numel() * t.element_size()
-    call("hipattn_stream_probe", modes[mode], dst.data_ptr() if dst is not None else None,
-         src.data_ptr() if src is not None else None, nbytes,
-         chunks.data_ptr() if chunks is not None else None, chunks.numel() if chunks is not None else 0, _stream(t))
-
-
 # --------------------------------------------------------------------------- runtime plumbing
 
 class Stats:

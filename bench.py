@@ -10,6 +10,7 @@ repeated until at least 100 ms have been timed; `value` is the median block, the
 The same line carries the other configurations: `prefill` (8 x 4096 GQA causal varlen prefill,
 TFLOP/s against the bf16 MFMA peak, with its own CPU baseline), `mixed_step` (the Phi-2-shaped
 continuous-batching step), `llama_step` (the full Llama-3-8B-shaped decode step with the AICI mask),
+`decode_c5_shape` (that step's decode attention alone, one layer, against the HBM roofline),
 `memory_system` (what plain read / copy / fill kernels reach on this device) and `cpu_baseline`
 (the oracle, i.e. rLLM's CPU reference route restated in torch-CPU, timed on a bounded sample of
 the decode workload on this box's host cores).
@@ -68,13 +69,16 @@ def spread(xs: list) -> dict:
 
 
 def host_cores() -> dict:
-    """Cores this process may run on and cores the box reports (a container's share can be smaller)."""
+    """Cores this process may run on and cores the box reports (a container's share can be smaller); the CPU
+    baselines run on every core the process may use, up to the thread count the box sets for such pools
+    (OMP_NUM_THREADS), and say how many that was."""
     try:
         usable = len(os.sched_getaffinity(0))
     except AttributeError:
         usable = os.cpu_count() or 1
-    # a one-GPU box of this pool shares its host: 16 cores go with one GPU, whatever the counts above say
-    return {"usable": usable, "reported": os.cpu_count() or 1, "share_for_one_gpu": 16, "threads_used": min(usable, 16)}
+    cap = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    threads = min(usable, cap) if cap > 0 else usable
+    return {"usable": usable, "reported": os.cpu_count() or 1, "omp_num_threads": cap or None, "threads_used": max(1, threads)}
 
 
 def cpu_baseline_prefill(p_cpu, seq: int, threads: int) -> dict:
@@ -169,7 +173,7 @@ def memory_system_leg(dev, stream, steps: int) -> dict:
     grid-stride), beside the published 8 TB/s: a 1 GiB read, a 1 GiB copy, a 1 GiB fill, and the read of
     a 1.3 GB buffer in shuffled 4 KiB chunks -- the granule and footprint of the decode leg's K/V blocks."""
     import torch
-    from aici_amd import kernels as K
+    from aici_amd import membench
 
     n = 1 << 30
     src = torch.empty((n,), dtype=torch.uint8, device=dev).fill_(1)
@@ -187,10 +191,16 @@ def memory_system_leg(dev, stream, steps: int) -> dict:
         ms = sum(ts) / len(ts)
         out[name] = {"GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1), "us": round(ms * 1e3, 1), "bytes": nbytes}
 
-    run("read_1GiB", lambda: K.stream_probe("read", None, src), n)
-    run("copy_1GiB_read_plus_write", lambda: K.stream_probe("copy", dst, src), 2 * n)
-    run("fill_1GiB", lambda: K.stream_probe("fill", dst, None), n)
-    run("read_4KiB_chunks_shuffled", lambda: K.stream_probe("read_chunks", None, big, order), order.numel() * 4096)
+    run("read_1GiB", lambda: membench.probe("read", None, src), n)
+    run("copy_1GiB_read_plus_write", lambda: membench.probe("copy", dst, src), 2 * n)
+    run("fill_1GiB", lambda: membench.probe("fill", dst, None), n)
+    run("read_4KiB_chunks_shuffled", lambda: membench.probe("read_chunks", None, big, order), order.numel() * 4096)
+    # the same amount in larger granules: what reading several kv heads of a block as one piece could give
+    for kib in (16, 32):
+        cb = kib * 1024
+        order_k = torch.randperm(big.numel() // cb, generator=g)[:154_000 * 4096 // cb].to(torch.int32).to(dev)
+        run(f"read_{kib}KiB_chunks_shuffled", lambda: membench.probe("read_chunks", None, big, order_k, cb),
+            order_k.numel() * cb)
     return out
 
 
@@ -310,7 +320,68 @@ def mixed_step_leg(dev, stream, steps: int) -> dict:
         torch.cuda.synchronize()
         ms = event_times_ms(fn, steps, stream)
         out[name] = {"us_per_step": round(sum(ms) / len(ms) * 1e3, 1)}
+    # The two attention kernels of the step on their own (the same calls the composition makes, on the cache the
+    # step above has filled), each against its roofline: the chunks against the fp16 MFMA peak, the decode rows
+    # against the HBM peak.
+    from aici_amd import kernels as K
+    scale = 1.0 / math.sqrt(d)
+    qm = q[:bi.q_multi]
+    chunks = lambda: K.flash_attn_varlen_paged(qm, kc, vc, bi.multi_block_tables, bi.seqlens_q, bi.multi_context_lens,
+                                               bi.max_seqlen_q, bi.max_seqlen_k, scale, True)
+    qd, o_d = q[bi.q_multi:], torch.empty_like(q[bi.q_multi:])
+    rows = lambda: K.paged_attention_v1(o_d, qd, kc, vc, H, scale, bi.paged_block_tables, bi.paged_context_lens, 16,
+                                        bi.paged_max_context_len)
+    dec_bytes = kv_bytes + 2 * len(dec) * H * d * 2 + 4 * sum((c + 15) // 16 for c in dec) + 4 * len(dec)
+    for fn in (chunks, rows):
+        for _ in range(10):
+            fn()
+    torch.cuda.synchronize()
+    ms_c = event_blocks_ms(chunks, max(steps, 10), stream)
+    ms_r = event_blocks_ms(rows, max(steps, 10), stream)
+    import statistics
+    mc, mr = statistics.median(ms_c), statistics.median(ms_r)
+    out["prefill_chunks"] = {"us": round(mc * 1e3, 1), "roofline": {
+        "bound": "mfma", "achieved": round(flops / (mc * 1e-3) / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(flops / (mc * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+        "kernel": "hipattn_mha_varlen_fwd_paged (block images), 4 x 512 rows, d 80 in the 96-wide instance"}}
+    out["decode_rows"] = {"us": round(mr * 1e3, 1), "algorithmic_bytes": dec_bytes, "roofline": {
+        "bound": "hbm", "achieved": round(dec_bytes / (mr * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(dec_bytes / (mr * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+        "kernel": "paged_attention_v1, whole call (main + merge kernel), 120 rows, MHA d 80"}}
     return out
+
+
+def decode_c5_shape_leg(dev, stream, steps: int) -> dict:
+    """The decode attention of the full-model configuration at its own shape, one layer: 128 sequences with
+    contexts U[1024, 16384] (seed 5), 32 q / 8 kv heads, d 128, bf16, block tables over a shuffled pool -- the
+    whole `paged_attention_v1` call (main + merge kernel) as algorithmic HBM GB/s."""
+    import statistics
+
+    import numpy as np
+    import torch
+
+    from aici_amd import kernels as K
+    from aici_amd import workloads as W
+
+    rng = np.random.default_rng(5)
+    S = 128
+    ctx = rng.integers(1024, 16384 + 1, size=S)
+    pool = int(((ctx + 15) // 16).sum()) + 64
+    c = W.decode_inputs(5, S, 1024, 16384, 32, 8, 128, torch.bfloat16, pool, device=dev)
+    out = torch.empty_like(c.q)
+    fn = lambda: K.paged_attention_v1(out, c.q, c.key_cache, c.value_cache, 8, c.scale, c.block_tables, c.context_lens,
+                                      16, c.max_ctx)
+    for _ in range(5):
+        fn()
+    torch.cuda.synchronize()
+    ms = statistics.median(event_blocks_ms(fn, max(steps, 10), stream))
+    nbytes = c.algorithmic_bytes()
+    return {"us_per_step": round(ms * 1e3, 1), "algorithmic_bytes": nbytes,
+            "roofline": {"bound": "hbm", "achieved": round(nbytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                         "kernel": "paged_attention_v1, whole call (main + merge kernel)"},
+            "config": {"workload": "paged decode attention, 128 seqs, ctx U[1024,16384] (seed 5), 32q/8kv heads, d128, "
+                                   "bf16, block 16, one layer", "context_tokens": int(ctx.sum())}}
 
 
 def llama_step_leg(dev, stream, steps: int, layers: int, share_cache: bool) -> dict:
@@ -418,6 +489,8 @@ def main() -> None:
     ap.add_argument("--no-llama-step", action="store_true",
                     help="skip the full Llama-3-8B-shaped decode step with the AICI mask + greedy stage "
                          "(it allocates about 170 GB of HBM)")
+    ap.add_argument("--no-decode-c5-shape", action="store_true",
+                    help="skip the decode attention of the full-model configuration at its own shape (one layer)")
     ap.add_argument("--mixed-step", action="store_true", help="(default; kept for old command lines)")
     ap.add_argument("--llama-step", action="store_true", help="(default; kept for old command lines)")
     ap.add_argument("--llama-layers", type=int, default=32)
@@ -586,6 +659,9 @@ def main() -> None:
 
     if not args.no_mixed_step:
         line["mixed_step"] = mixed_step_leg(dev, stream, max(100, args.steps))
+
+    if not args.no_decode_c5_shape:
+        line["decode_c5_shape"] = decode_c5_shape_leg(dev, stream, args.steps)
 
     # ---- the full engine step the decode kernel sits in -------------------------------------------
     if not args.no_llama_step:

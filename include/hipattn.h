@@ -385,15 +385,6 @@ char *hipattn_empty_cache(void); /* nothing to release: no caching allocator; se
 char *hipattn_get_stats_allocated_bytes(int device, hipattn_mem_stats *outp);
 char *hipattn_get_device_properties(int device, hipattn_device_props *outp);
 
-/* No counterpart in the reference: yardsticks for the memory system, for benchmark harnesses that want
- * the attainable streaming rates of the device beside a kernel's own figure.  One launch on `stream`:
- * mode 0 reads `bytes` from src once (dst: NULL or 4 bytes of device memory, never written in practice),
- * mode 1 copies src to dst, mode 2 fills dst, mode 3 reads the 4 KiB chunks of src that `chunks[0..n_chunks)`
- * number (each 0 <= chunks[k] < bytes / 4096) -- the granule in which the paged caches are read.  bytes
- * must be a multiple of 16 (4096 for mode 3). */
-char *hipattn_stream_probe(int mode, void *dst, const void *src, int64_t bytes, const int32_t *chunks,
-                           int64_t n_chunks, void *stream);
-
 typedef struct hipattn_stream hipattn_stream;
 typedef struct hipattn_event hipattn_event;
 

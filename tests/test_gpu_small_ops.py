@@ -389,24 +389,26 @@ def test_streams_events_and_memory_figures(device):
     s.synchronize()
 
 
-def test_stream_probe_modes(device):
-    """The memory-system yardsticks: copy and fill do what they say, the reads launch and leave their
-    source alone, bad arguments come back as messages."""
+def test_memory_yardsticks_of_the_benchmark(device):
+    """The benchmark's memory-system yardsticks (a library of their own, libmembench.so): copy and fill do
+    what they say, the reads launch and leave their source alone, bad arguments are refused."""
+    from aici_amd import membench
     g = torch.Generator().manual_seed(5)
     src = torch.randint(0, 255, (8 * 4096 + 16,), generator=g, dtype=torch.uint8).to(device)
     dst = torch.zeros_like(src)
-    K.stream_probe("copy", dst, src)
+    membench.probe("copy", dst, src)
     assert torch.equal(dst.cpu(), src.cpu())
-    K.stream_probe("fill", dst, None)
+    membench.probe("fill", dst, None)
     want = torch.tensor([1, 2, 3, 4], dtype=torch.int32).repeat(dst.numel() // 16)
     assert torch.equal(dst.cpu().view(torch.int32), want)
     before = src.cpu().clone()
-    K.stream_probe("read", None, src)
+    membench.probe("read", None, src)
     chunks = torch.tensor([7, 0, 3, 3, 5], dtype=torch.int32, device=device)
-    K.stream_probe("read_chunks", None, src[: 8 * 4096], chunks)
+    membench.probe("read_chunks", None, src[: 8 * 4096], chunks)
+    membench.probe("read_chunks", None, src[: 8 * 4096], torch.tensor([1, 0], dtype=torch.int32, device=device), 16384)
     torch.cuda.synchronize()
     assert torch.equal(src.cpu(), before)
-    with pytest.raises(HipAttnError, match="multiple of 16"):
-        K.stream_probe("read", None, src[:100])
-    with pytest.raises(HipAttnError, match="multiple of 4096"):
-        K.stream_probe("read_chunks", None, src, chunks)
+    with pytest.raises(RuntimeError, match="bad arguments"):
+        membench.probe("read", None, src[:100])
+    with pytest.raises(RuntimeError, match="bad arguments"):
+        membench.probe("read_chunks", None, src[: 4096 + 16], chunks)
