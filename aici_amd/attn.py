@@ -74,7 +74,7 @@ def varlen_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, batch_info: B
     gather, varlen prefill rows, paged decode rows) is one C-ABI call.  With
     `paged_prefill` the multi-token rows read their context from the cache
     through block tables instead of a gathered copy (needs the builder's
-    multi_block_tables and d <= 128)."""
+    multi_block_tables)."""
     T, Hq, d = q.shape
     Hkv = k.size(1)
     if softmax_scale is None:

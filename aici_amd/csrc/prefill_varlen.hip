@@ -63,13 +63,18 @@ struct Tile {
   static constexpr int VSTR = (HDP % 64 == 32) ? HDP : HDP + 32;
   static constexpr int K_ELEMS = BN * KSTR;
   static constexpr int V_ELEMS = BN * VSTR;
-  static constexpr int STAGE_ELEMS = K_ELEMS + V_ELEMS;
+  static constexpr int VTSTR = BN + 8;  // paged form: V^T rows (head-element-major), 64 keys + 16 B
+  static constexpr int VT_ELEMS = HDP * VTSTR;
+  static constexpr int STAGE_ELEMS = K_ELEMS + (V_ELEMS > VT_ELEMS ? V_ELEMS : VT_ELEMS);
   static constexpr size_t LDS_BYTES = 2 * (size_t)STAGE_ELEMS * 2;
 };
 
 typedef __attribute__((address_space(3))) s16x4_t lds_s16x4;
 
-template <typename T, int HDP, int QT>
+// PAGED: K and V are the paged caches, read through the block table (p.block_tables, p.context_lens); tiles
+// are staged in the caches' own order -- 16-byte runs of K go to the rows they belong to, 16-byte runs of V (8
+// tokens of one head element) to rows of a V^T tile, whose operands plain 8-byte LDS reads deliver.
+template <typename T, int HDP, int QT, bool PAGED = false>
 __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
   typedef typename Vec8<T>::type vec8;
   typedef Tile<HDP> TL;
@@ -100,9 +105,9 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
 
   const int q_begin = p.cu_q[b];
   const int Lq = p.cu_q[b + 1] - q_begin;
-  const int k_begin = p.cu_k[b];
-  int Lk = p.cu_k[b + 1] - k_begin;
-  if (p.seqused_k) Lk = min(Lk, p.seqused_k[b]);
+  const int k_begin = PAGED ? 0 : p.cu_k[b];
+  int Lk = PAGED ? p.context_lens[b] : p.cu_k[b + 1] - k_begin;
+  if (!PAGED && p.seqused_k) Lk = min(Lk, p.seqused_k[b]);
   const int wg_row0 = qb * BM;
   if (wg_row0 >= Lq) return;
   const int off = Lk - Lq;  // bottom-right alignment of the mask
@@ -118,8 +123,8 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
   const int wave_last_row = wave_row0 + QT * 32 - 1;
 
   const T *qp = static_cast<const T *>(p.q) + (int64_t)q_begin * p.q_row + (int64_t)h * p.q_head;
-  const T *kp = static_cast<const T *>(p.k) + (int64_t)k_begin * p.k_row + (int64_t)kvh * p.k_head;
-  const T *vp = static_cast<const T *>(p.v) + (int64_t)k_begin * p.v_row + (int64_t)kvh * p.v_head;
+  const T *kp = static_cast<const T *>(p.k) + (PAGED ? (int64_t)kvh * p.kc_head : (int64_t)k_begin * p.k_row + (int64_t)kvh * p.k_head);
+  const T *vp = static_cast<const T *>(p.v) + (PAGED ? (int64_t)kvh * p.vc_head : (int64_t)k_begin * p.v_row + (int64_t)kvh * p.v_head);
   const int d_chunks = p.d / 8;
 
   // Q operands: lane (g, c) of tile qt holds q[row][16ks + 8g .. +8].
@@ -152,8 +157,39 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
 
   // Tile staging: thread t moves chunk (t + 256 i) of the tile.
   u32x4_t kst[NLOAD], vst[NLOAD];
+  int staged_k0 = 0;  // first key of the tile held in the staging registers (paged form)
+  const int32_t *table_row = PAGED ? p.block_tables + (int64_t)b * p.table_stride : nullptr;
   auto load_tile = [&](int tile) {
     const int k0 = tile * BN;
+    if constexpr (PAGED) {
+      // Units in the caches' own order, so that consecutive threads read consecutive 16-byte runs: K unit
+      // (block r, chunk, token), V unit (block r, head element, half of the block's tokens).  Blocks past the
+      // context re-read its last one (their keys are masked, their V runs cleared before they reach LDS).
+      staged_k0 = k0;
+      const int last_col = max(min((Lk - 1) >> 4, p.table_cols - 1), 0);
+      int64_t blk[4];
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int id = table_row[min((k0 >> 4) + r, last_col)];
+        blk[r] = id < 0 ? 0 : (id >= p.num_blocks ? p.num_blocks - 1 : (int64_t)id);
+      }
+      constexpr int K_PER_BLOCK = CPR * 16, V_PER_BLOCK = HDP * 2;
+#pragma unroll
+      for (int i = 0; i < NLOAD; i++) {
+        const int u = tid + 256 * i;
+        {
+          const int r = u / K_PER_BLOCK, rem = u % K_PER_BLOCK;
+          const int ch = min(rem / 16, d_chunks - 1), tok = rem % 16;
+          kst[i] = *reinterpret_cast<const u32x4_t *>(kp + blk[r] * p.kc_block + (ch * 16 + tok) * 8);
+        }
+        {
+          const int r = u / V_PER_BLOCK, rem = u % V_PER_BLOCK;
+          const int drow = min(rem / 2, p.d - 1), half = rem % 2;
+          vst[i] = *reinterpret_cast<const u32x4_t *>(vp + blk[r] * p.vc_block + drow * 16 + half * 8);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NLOAD; i++) {
       const int idx = tid + 256 * i;
@@ -170,6 +206,35 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
   auto store_tile = [&](int stage) {
     T *ks = smem + stage * TL::STAGE_ELEMS;
     T *vs = ks + TL::K_ELEMS;
+    if constexpr (PAGED) {
+      constexpr int K_PER_BLOCK = CPR * 16, V_PER_BLOCK = HDP * 2;
+#pragma unroll
+      for (int i = 0; i < NLOAD; i++) {
+        const int u = tid + 256 * i;
+        {
+          const int r = u / K_PER_BLOCK, rem = u % K_PER_BLOCK;
+          // (chunks past d carry a copy of the last real one: they meet the zeros of Q)
+          *reinterpret_cast<u32x4_t *>(ks + (r * 16 + rem % 16) * TL::KSTR + (rem / 16) * 8) = kst[i];
+        }
+        {
+          const int r = u / V_PER_BLOCK, rem = u % V_PER_BLOCK;
+          const int drow = rem / 2, half = rem % 2;
+          u32x4_t o = vst[i];
+          // Cache tokens past the context hold whatever was there before (possibly NaN, which a zero
+          // probability would not neutralise): clear them.
+          if (staged_k0 + BN > Lk) {
+            const int alive = Lk - (staged_k0 + r * 16 + half * 8);  // keys of this run inside the context
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+              const int a2 = alive - 2 * w;
+              o[w] &= a2 <= 0 ? 0u : (a2 == 1 ? 0xffffu : 0xffffffffu);
+            }
+          }
+          *reinterpret_cast<u32x4_t *>(vs + drow * TL::VTSTR + r * 16 + half * 8) = o;
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NLOAD; i++) {
       const int idx = tid + 256 * i;
@@ -282,9 +347,17 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
         for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
           for (int half = 0; half < 2; half++) {
-            const T *vptr = vs_base + v_lane_off + (hf * 32 + half * 16) * TL::VSTR + dt * 32;
-            const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vptr));
-            const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vptr + 8 * TL::VSTR));
+            s16x4_t lo, hi;
+            if constexpr (PAGED) {
+              // V^T rows: head element dt * 32 + c, keys 4 g .. + 4 of the 16-key step and 8 further on
+              const T *vptr = vs_base + (dt * 32 + c) * TL::VTSTR + hf * 32 + half * 16 + 4 * g;
+              lo = *reinterpret_cast<const s16x4_t *>(vptr);
+              hi = *reinterpret_cast<const s16x4_t *>(vptr + 8);
+            } else {
+              const T *vptr = vs_base + v_lane_off + (hf * 32 + half * 16) * TL::VSTR + dt * 32;
+              lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vptr));
+              hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vptr + 8 * TL::VSTR));
+            }
             typedef short s16x8 __attribute__((ext_vector_type(8)));
             const s16x8 av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             const vec8 a = bit_cast<vec8>(av);
@@ -1243,11 +1316,11 @@ void launch_prefill_w8(PrefillParams p, hipStream_t stream) {
   check_launch("mha_varlen_fwd");
 }
 
-template <typename T, int HDP, int QT>
+template <typename T, int HDP, int QT, bool PAGED = false>
 void launch_prefill(PrefillParams p, hipStream_t stream) {
   constexpr int BM = 4 * QT * 32;
   static bool attr_set = false;  // benign race: setting twice is harmless
-  auto kernel = prefill_varlen_kernel<T, HDP, QT>;
+  auto kernel = prefill_varlen_kernel<T, HDP, QT, PAGED>;
   if (!attr_set) {
     HA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)Tile<HDP>::LDS_BYTES));
@@ -1426,7 +1499,7 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
 
 // Varlen prefill whose keys and values are read from the paged cache through block tables: what
 // rLLM composes from gather_cached_kv -> repeat_kv -> flash_attn_varlen (llm/mod.rs:181-238) without
-// the two copies.  Eight-wavefront kernel only (head sizes up to 128).
+// the two copies.  Eight-wavefront kernel for head sizes up to 128, four-wavefront kernel above.
 template <typename T>
 void dispatch_paged(const PrefillParams &p, hipStream_t stream) {
   const int hdp = ((p.d + 31) / 32) * 32;
@@ -1444,7 +1517,12 @@ void dispatch_paged(const PrefillParams &p, hipStream_t stream) {
     case 64: HA_W8P(64); break;
     case 96: HA_W8P(96); break;
     case 128: HA_W8P(128); break;
-    default: fail("mha_varlen_fwd_paged: head size %d not supported (at most 128)", p.d);
+    // head sizes above 128: the four-wavefront kernel, tiles staged through registers
+    case 160: launch_prefill<T, 160, 1, true>(p, stream); break;
+    case 192: launch_prefill<T, 192, 1, true>(p, stream); break;
+    case 224: launch_prefill<T, 224, 1, true>(p, stream); break;
+    case 256: launch_prefill<T, 256, 1, true>(p, stream); break;
+    default: fail("mha_varlen_fwd_paged: head size %d not supported (at most 256)", p.d);
   }
 #undef HA_W8P
 }
@@ -1459,7 +1537,7 @@ void mha_varlen_fwd_paged_impl(const hipattn_tensor *q, const hipattn_tensor *ke
            dtype_name(q->dtype));
   const int d = (int)q->sizes[2];
   const int Hq = (int)q->sizes[1];
-  HA_CHECK(d % 8 == 0 && d > 0 && d <= 128, "%s: head size must be a multiple of 8 in (0, 128], got %d", op, d);
+  HA_CHECK(d % 8 == 0 && d > 0 && d <= 256, "%s: head size must be a multiple of 8 in (0, 256], got %d", op, d);
   check_qkv(q, "q", q->dtype, d);
   check_qkv(out, "out", q->dtype, d, true);
   HA_CHECK(out->sizes[0] == q->sizes[0] && out->sizes[1] == Hq, "%s: out shape differs from q", op);

@@ -101,7 +101,8 @@ char *hipattn_mha_varlen_fwd(const hipattn_tensor *q, const hipattn_tensor *k,
  * is in block block_tables[i][p / 16] at offset p % 16 (the new tokens' K/V
  * must already be in the cache); cu_seqlens_q int32 [b+1]; context_lens int32
  * [b] = keys per sequence; causal mask bottom-right aligned as in
- * hipattn_mha_varlen_fwd; out in q's dtype or f32 as there.  fp16/bf16, d % 8 == 0, d <= 128, block size 16. */
+ * hipattn_mha_varlen_fwd; out in q's dtype or f32 as there.  fp16/bf16, d % 8 == 0, d <= 256 (what
+ * flash_api.cpp:522-523 serves), block size 16. */
 char *hipattn_mha_varlen_fwd_paged(const hipattn_tensor *q, const hipattn_tensor *key_cache,
                                    const hipattn_tensor *value_cache, const hipattn_tensor *block_tables,
                                    const hipattn_tensor *cu_seqlens_q, const hipattn_tensor *context_lens,
@@ -660,7 +661,7 @@ char *hipattn_varlen_attn(
  * context from the cache through multi_block_tables int32 [num_multi, cols] and
  * multi_context_lens int32 [num_multi] (hipattn_mha_varlen_fwd_paged).  No
  * counterpart in the reference, which always gathers (mod.rs:181-197).  Head
- * sizes up to 128. */
+ * sizes up to 256. */
 char *hipattn_varlen_attn_paged(
     const hipattn_tensor *q, const hipattn_tensor *k, const hipattn_tensor *v,
     hipattn_tensor *key_cache, hipattn_tensor *value_cache,

@@ -19,10 +19,10 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(autouse=True, params=["auto", "staged"])
 def tile_route(request, tuning):
-    """Head sizes from 40 up (and 32) have their tiles copied from the cache into LDS as block images -- those
-    that do not fill their MFMA tiles (40, 72, 80, 104, ...) with the rest of each image's place cleared; the
-    smaller ones -- and every size when the tuning switch paged_prefill_dma is 0 -- are staged through
-    registers.  Every test runs both ways."""
+    """Head sizes from 40 up to 128 (and 32) have their tiles copied from the cache into LDS as block images --
+    those that do not fill their MFMA tiles (40, 72, 80, 104, ...) with the rest of each image's place cleared;
+    the smaller ones -- and every size when the tuning switch paged_prefill_dma is 0 -- are staged through
+    registers, as are head sizes above 128, which the four-wavefront kernel takes.  Every test runs both ways."""
     tuning("paged_prefill_dma", -1 if request.param == "auto" else 0)
     return request.param
 
@@ -76,7 +76,8 @@ SEQS = [(0, 5), (0, 64), (100, 33), (1000, 256), (17, 1), (0, 300), (63, 65), (2
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("heads", [(32, 8, 128), (32, 32, 80), (8, 2, 64), (4, 4, 32), (6, 1, 96), (8, 2, 112), (4, 4, 120),
-                                   (4, 2, 8), (4, 2, 40), (4, 4, 72), (2, 1, 104)])
+                                   (4, 2, 8), (4, 2, 40), (4, 4, 72), (2, 1, 104),
+                                   (4, 2, 160), (4, 4, 192), (2, 1, 200), (8, 2, 256)])
 def test_matches_oracle(device, dtype, heads):
     Hq, Hkv, d = heads
     c = paged_case(31, SEQS, Hq, Hkv, d, dtype, 420)
@@ -128,7 +129,7 @@ def test_random_ragged_cases(device):
     pick = lambda xs: xs[int(rng.integers(len(xs)))]
     for case in range(16):
         dtype = pick([torch.bfloat16, torch.float16])
-        d = pick([32, 40, 64, 80, 96, 120, 128])
+        d = pick([32, 40, 64, 80, 96, 120, 128, 160, 256])
         Hkv = pick([1, 2, 4])
         Hq = Hkv * pick([1, 2, 4])
         seqs = [(pick([0, 0, 7, 16, 64, 100, 333, 700]), pick([1, 5, 15, 16, 17, 63, 64, 65, 255, 257, 513]))
@@ -181,7 +182,7 @@ def test_argument_errors(device):
         K.flash_attn_varlen_paged(c["q"].to(device), c["kc"].to(device), c["vc"].to(device), c["tables"].to(device),
                                   c["cu_q"].to(device), c["ctx"].to(device), 20, 16 * c["tables"].size(1) + 1,
                                   c["scale"], True)
-    big = paged_case(35, [(0, 4)], 2, 2, 256, torch.float16, 4)
+    big = paged_case(35, [(0, 4)], 2, 2, 264, torch.float16, 4)
     with pytest.raises(HipAttnError, match="head size"):
         run_paged(big, device)
 
