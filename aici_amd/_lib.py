@@ -146,6 +146,10 @@ _ERR_FUNCS = {
     "hipattn_block_allocator_step_generation": [c_void_p, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), c_int64,
                                                 POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
                                                 POINTER(c_int64), c_int64, POINTER(c_int64)],
+    "hipattn_block_space_step_generation": [c_void_p, c_void_p, c_int64, POINTER(c_int64), POINTER(c_int64),
+                                            POINTER(c_int64), POINTER(c_int32), POINTER(c_int64), POINTER(c_int64),
+                                            POINTER(c_int32), POINTER(c_int64), c_int64, POINTER(c_int64),
+                                            POINTER(c_int64), c_int64, POINTER(c_int64)],
     "hipattn_varlen_attn": [TP, TP, TP, TP, TP, TP, TP, TP, TP, c_int64, c_int, c_int, TP, TP, c_int, c_int, c_float,
                             TP, TP, TP, c_void_p],
     "hipattn_varlen_attn_paged": [TP, TP, TP, TP, TP, TP, TP, TP, TP, c_int64, c_int, c_int, TP, TP, c_int, c_int,

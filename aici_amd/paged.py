@@ -117,6 +117,11 @@ class BlockAllocator:
             mapping[int(pairs[2 * i])] = int(pairs[2 * i + 1])
 
 
+# SchedulingPhase (seq.rs:44-51) and what `BlockSpaceManager.step_generation` did with a group.
+SEQ_RUNNING, SEQ_SUSPENDED, SEQ_SWAPPED, SEQ_WAITING, SEQ_FINISHED = range(5)
+GROUP_NOT_REACHED, GROUP_SCHEDULED, GROUP_SUSPENDED, GROUP_RECOMPUTE, GROUP_SWAPPED_OUT = -1, 0, 1, 2, 3
+
+
 class BlockSpaceManager:
     """blocks.rs:259-380: the mapping between logical and physical blocks on both sides of the swap --
     a device allocator with its admission watermark and a host allocator.  Sequences are plain ids;
@@ -174,6 +179,36 @@ class BlockSpaceManager:
         for s in running_seq_ids:
             self.cpu_allocator.swap_in(s, self.gpu_allocator.swap_out(s), mapping)
         return mapping
+
+    def step_generation(self, groups: Sequence[Tuple[int, Sequence[Tuple[int, int, int, int]]]]) -> dict:
+        """scheduler.rs:304-337, 346-380 for sequence groups of any size.  groups, in arrival order, are
+        (max_running_seqs, [(seq_id, phase, seq_len to grow to, num_kv_computed), ...]) with phase one of
+        SEQ_RUNNING .. SEQ_FINISHED.  Returns {"fates": one GROUP_* per group, "copies": copy-on-write
+        (old, new) device block pairs, "swap_out": (device block, host block) pairs for
+        `CacheEngine.swap_out`}."""
+        starts, ids, phases, lens, comp, maxrun = [0], [], [], [], [], []
+        for max_running, seqs in groups:
+            maxrun.append(int(max_running))
+            for sid, phase, seq_len, computed in seqs:
+                ids.append(int(sid))
+                phases.append(int(phase))
+                lens.append(int(seq_len))
+                comp.append(int(computed))
+            starts.append(len(ids))
+        g, n = len(maxrun), len(ids)
+        bs = self.gpu_allocator.block_size
+        cap_copy = sum((l + bs - 1) // bs + 1 for l in lens) + 1
+        cap_swap = sum(self.gpu_allocator.num_allocated_blocks(s) for s in ids) + 1
+        a64 = lambda v: (ctypes.c_int64 * max(1, len(v)))(*v)
+        fates = (ctypes.c_int32 * max(1, g))()
+        copies, swaps = (ctypes.c_int64 * (2 * cap_copy))(), (ctypes.c_int64 * (2 * cap_swap))()
+        nc, nsw = ctypes.c_int64(), ctypes.c_int64()
+        call("hipattn_block_space_step_generation", self.gpu_allocator._h, self.cpu_allocator._h, g, a64(starts),
+             a64(maxrun), a64(ids), (ctypes.c_int32 * max(1, n))(*phases), a64(lens), a64(comp), fates, copies,
+             cap_copy, ctypes.byref(nc), swaps, cap_swap, ctypes.byref(nsw))
+        return {"fates": [int(fates[i]) for i in range(g)],
+                "copies": [(int(copies[2 * i]), int(copies[2 * i + 1])) for i in range(nc.value)],
+                "swap_out": [(int(swaps[2 * i]), int(swaps[2 * i + 1])) for i in range(nsw.value)]}
 
     def get_num_free_gpu_blocks(self) -> int:
         return self.gpu_allocator.get_num_free_blocks()

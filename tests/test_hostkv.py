@@ -425,3 +425,217 @@ def test_step_generation_matches_restatement(seed):
         assert a.get_num_free_blocks() == r.get_num_free_blocks()
         for s in running:
             assert a.get_block_idxes(s, lens[s]).tolist() == r.get_block_idxes(s, lens[s])
+
+
+def _space(bs, n_gpu, n_cpu):
+    m = paged.BlockSpaceManager(bs, n_gpu, n_cpu, watermark=0.0)
+    return m, ref.BlockAllocator(bs, n_gpu), ref.BlockAllocator(bs, n_cpu)
+
+
+def test_group_step_swaps_out_a_group_of_two_hand_case():
+    """8 device blocks of 4 tokens, all taken: group A = sequence 1 (blocks 0-2), group B = sequence 2 (3-5),
+    group C = sequences 3 and 4 which share blocks 6, 7 (a fork).  A needs one free block, so C, the latest
+    arrival, is preempted; it runs two sequences, so it is swapped: blocks 6, 7 go to host blocks 0, 1 -- once,
+    both sequences then hold host blocks [0, 1] -- and the device gets 6, 7 back (7 on top of the stack).  A takes
+    7, B takes 6."""
+    m, _, _ = _space(4, 8, 8)
+    g = m.gpu_allocator
+    g.alloc_seq(1, 12)
+    g.alloc_seq(2, 12)
+    g.alloc_seq(3, 8)
+    g.copy(3, 4, 8)
+    assert g.get_num_free_blocks() == 0
+    R = paged.SEQ_RUNNING
+    out = m.step_generation([(1, [(1, R, 13, 12)]), (1, [(2, R, 13, 12)]), (2, [(3, R, 9, 8), (4, R, 9, 8)])])
+    assert out["fates"] == [paged.GROUP_SCHEDULED, paged.GROUP_SCHEDULED, paged.GROUP_SWAPPED_OUT]
+    assert out["copies"] == [] and out["swap_out"] == [(6, 0), (7, 1)]
+    assert g.num_allocated_blocks(3) == 0 and g.num_allocated_blocks(4) == 0
+    c = m.cpu_allocator
+    assert list(c.get_block_idxes(3, 8)) == list(c.get_block_idxes(4, 8)) == list(range(8))
+    assert c.get_num_free_blocks() == 6 and g.get_num_free_blocks() == 0
+    assert g.get_block_idxes(1, 13)[-1] == 7 * 4 and g.get_block_idxes(2, 13)[-1] == 6 * 4
+    # the way back once there is room: the shared blocks stay shared
+    g.delete(1)
+    assert not m.can_swap_in([3, 4])   # the check counts a shared block once per holder, plus one per sequence
+    g.delete(2)
+    assert m.can_swap_in([3, 4])
+    back = m.swap_in([3, 4])
+    assert sorted(back) == [0, 1] and c.get_num_free_blocks() == 8
+    assert list(g.get_block_idxes(3, 8)) == list(g.get_block_idxes(4, 8))
+    assert g.get_num_free_blocks() == 6
+
+
+def test_group_step_suspended_groups_hand_case():
+    R, S, F = paged.SEQ_RUNNING, paged.SEQ_SUSPENDED, paged.SEQ_FINISHED
+    # the suspended group arrived first: it is set aside, so the running group finds nobody to preempt but itself
+    m, _, _ = _space(4, 4, 4)
+    m.gpu_allocator.alloc_seq(1, 8)
+    m.gpu_allocator.alloc_seq(2, 8)
+    out = m.step_generation([(1, [(1, S, 8, 8)]), (1, [(2, R, 9, 8)])])
+    assert out["fates"] == [paged.GROUP_SUSPENDED, paged.GROUP_RECOMPUTE]
+    assert m.gpu_allocator.num_allocated_blocks(1) == 2 and m.gpu_allocator.num_allocated_blocks(2) == 0
+    # the suspended group arrived last: it is still queued when a victim is needed.  With no running sequence it
+    # is not a group of one, so it goes the swap way, where only running sequences move: nothing is freed and
+    # the running group ends up preempting itself as well.
+    m, _, _ = _space(4, 4, 4)
+    m.gpu_allocator.alloc_seq(1, 8)
+    m.gpu_allocator.alloc_seq(2, 8)
+    out = m.step_generation([(1, [(1, R, 9, 8)]), (0, [(2, S, 8, 8)])])
+    assert out["fates"] == [paged.GROUP_RECOMPUTE, paged.GROUP_SWAPPED_OUT] and out["swap_out"] == []
+    assert m.gpu_allocator.num_allocated_blocks(2) == 2 and m.gpu_allocator.get_num_free_blocks() == 2
+    # with room for everybody a suspended group just stays; a finished sequence beside a suspended one counts
+    # as suspended, beside a running one it is skipped
+    m, _, _ = _space(4, 16, 4)
+    for s in (1, 2, 3, 4):
+        m.gpu_allocator.alloc_seq(s, 8)
+    out = m.step_generation([(2, [(1, S, 8, 8), (2, F, 8, 8)]), (2, [(3, R, 9, 8), (4, F, 8, 8)])])
+    assert out["fates"] == [paged.GROUP_SUSPENDED, paged.GROUP_SCHEDULED]
+    assert [m.gpu_allocator.num_allocated_blocks(s) for s in (1, 2, 3, 4)] == [2, 2, 3, 2]
+    # one free block per running sequence is asked for: two free blocks do not serve a group of three
+    m, _, _ = _space(4, 8, 8)
+    for s in (1, 2, 3):
+        m.gpu_allocator.alloc_seq(s, 8)
+    out = m.step_generation([(3, [(1, R, 9, 8), (2, R, 9, 8), (3, R, 9, 8)])])
+    assert out["fates"] == [paged.GROUP_SWAPPED_OUT] and len(out["swap_out"]) == 6
+    assert m.gpu_allocator.get_num_free_blocks() == 8 and m.cpu_allocator.get_num_free_blocks() == 2
+
+
+def test_group_step_errors():
+    R, F = paged.SEQ_RUNNING, paged.SEQ_FINISHED
+    m, _, _ = _space(4, 4, 1)
+    m.gpu_allocator.alloc_seq(1, 8)
+    m.gpu_allocator.alloc_seq(2, 4)
+    m.gpu_allocator.alloc_seq(3, 4)
+    with pytest.raises(HipAttnError, match="lack of CPU swap space"):
+        m.step_generation([(1, [(1, R, 9, 8)]), (2, [(2, R, 5, 4), (3, R, 5, 4)])])
+    # nothing moved: the check comes before the first block changes sides
+    assert m.gpu_allocator.get_num_free_blocks() == 0 and m.cpu_allocator.get_num_free_blocks() == 1
+    with pytest.raises(HipAttnError, match="has finished"):
+        m.step_generation([(1, [(1, R, 9, 8)]), (1, [(2, R, 5, 4), (3, F, 4, 4)])])
+    with pytest.raises(HipAttnError, match="phase"):
+        m.step_generation([(1, [(1, 7, 9, 8)])])
+    assert m.step_generation([]) == {"fates": [], "copies": [], "swap_out": []}
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_group_step_matches_restatement(seed):
+    """A scheduler's life in little: groups are admitted, fork inside themselves, get suspended for a step,
+    lose sequences, are swapped out and come back, or are dropped for recomputation and admitted again -- the
+    C++ core and the restatement are given the same calls and must agree on every answer and every table."""
+    rng = np.random.default_rng(900 + seed)
+    bs, n_gpu, n_cpu = 4, 48, 40
+    m, rg, rc = _space(bs, n_gpu, n_cpu)
+    R, S, F = paged.SEQ_RUNNING, paged.SEQ_SUSPENDED, paged.SEQ_FINISHED
+    on_gpu, swapped, waiting = [], [], []   # groups: {"best_of", "seqs": {id: len}, "finished": set}
+    next_id = 1
+    n_swaps = n_recomputes = 0
+
+    def same_state():
+        assert m.gpu_allocator.get_num_free_blocks() == rg.get_num_free_blocks()
+        assert m.cpu_allocator.get_num_free_blocks() == rc.get_num_free_blocks()
+        for grp in on_gpu + swapped:
+            for s, n in grp["seqs"].items():
+                for mine, theirs in ((m.gpu_allocator, rg), (m.cpu_allocator, rc)):
+                    k = theirs.num_allocated_blocks(s)
+                    assert mine.num_allocated_blocks(s) == k
+                    if k:
+                        assert list(mine.get_block_idxes(s, k * bs)) == theirs.get_block_idxes(s, k * bs)
+
+    for step in range(120):
+        # swapped groups come back first (step_swap_in), then prompts are admitted
+        while swapped:
+            grp = swapped[0]
+            ids = list(grp["seqs"])
+            want = sum(rc.num_allocated_blocks(s) for s in ids) + len(ids)
+            assert m.can_swap_in(ids) == (rg.get_num_free_blocks() >= want)
+            if not m.can_swap_in(ids):
+                break
+            got = m.swap_in(ids)
+            mapping = {}
+            for s in ids:
+                rg.swap_in(s, rc.swap_out(s), mapping)
+            assert got == mapping
+            on_gpu.append(swapped.pop(0))
+        while not swapped and rng.random() < 0.6:
+            if waiting and rng.random() < 0.7:
+                grp = waiting[0]
+            else:
+                grp = {"best_of": int(rng.choice([1, 1, 2, 3])), "seqs": {next_id: int(rng.integers(1, 30))},
+                       "finished": set()}
+                next_id += 1
+            (sid, n), = grp["seqs"].items()
+            assert m.can_allocate(n) == rg.can_allocate(n)
+            if not rg.can_allocate(n):
+                break
+            m.allocate(sid, n)
+            rg.alloc_seq(sid, n)
+            if waiting and grp is waiting[0]:
+                waiting.pop(0)
+            on_gpu.append(grp)
+        # after its prompt a group of best_of > 1 forks up to that many sequences
+        for grp in on_gpu:
+            live = [s for s in grp["seqs"] if s not in grp["finished"]]
+            if live and len(grp["seqs"]) < grp["best_of"] and rng.random() < 0.5:
+                src = live[int(rng.integers(len(live)))]
+                m.gpu_allocator.copy(src, next_id, grp["seqs"][src])
+                rg.copy(src, next_id, grp["seqs"][src])
+                grp["seqs"][next_id] = grp["seqs"][src]
+                next_id += 1
+        # a sequence of a group finishes now and then; its blocks go
+        for grp in list(on_gpu):
+            live = [s for s in grp["seqs"] if s not in grp["finished"]]
+            if live and rng.random() < 0.08:
+                s = live[int(rng.integers(len(live)))]
+                grp["finished"].add(s)
+                m.gpu_allocator.delete(s)
+                rg.delete(s)
+                if len(grp["finished"]) == len(grp["seqs"]):
+                    on_gpu.remove(grp)
+        same_state()
+        # the generation step
+        on_gpu.sort(key=lambda grp: min(grp["seqs"]))     # arrival = first id handed out
+        groups = []
+        for grp in on_gpu:
+            susp = rng.random() < 0.15
+            seqs = []
+            for s, n in grp["seqs"].items():
+                ph = F if s in grp["finished"] else (S if susp else R)
+                seqs.append((s, ph, n + 1, n))
+            running = sum(ph == R for _, ph, _, _ in seqs)
+            max_running = grp["best_of"] if grp["best_of"] > len(seqs) else running     # seq.rs:275-292
+            groups.append((max_running, seqs))
+        try:
+            want = ref.step_generation_groups(rg, rc, groups)
+        except (ref.OutOfBlocks, AssertionError):
+            with pytest.raises(HipAttnError):
+                m.step_generation(groups)
+            break
+        got = m.step_generation(groups)
+        assert got["fates"] == want[0] and got["copies"] == want[1] and got["swap_out"] == want[2]
+        keep = []
+        for grp, (_, seqs), fate in zip(on_gpu, groups, got["fates"]):
+            if fate == paged.GROUP_SCHEDULED:
+                for s, ph, n1, _ in seqs:
+                    if ph == R:
+                        grp["seqs"][s] = n1
+                keep.append(grp)
+            elif fate == paged.GROUP_SUSPENDED:
+                keep.append(grp)
+            elif fate == paged.GROUP_SWAPPED_OUT:
+                if any(ph == R for _, ph, _, _ in seqs):
+                    n_swaps += 1
+                    grp["seqs"] = {s: n for s, n in grp["seqs"].items() if s not in grp["finished"]}
+                    grp["finished"] = set()
+                    swapped.append(grp)
+                else:
+                    keep.append(grp)      # nothing moved: the group still sits on the device
+            elif fate == paged.GROUP_RECOMPUTE:
+                n_recomputes += 1
+                first = min(grp["seqs"])
+                grp["seqs"] = {first: grp["seqs"][first]}     # back to a prompt of one sequence
+                waiting.append(grp)
+            else:
+                keep.append(grp)          # not reached: the walk ended before it
+        on_gpu = keep
+        same_state()
+    assert n_swaps + n_recomputes > 0
