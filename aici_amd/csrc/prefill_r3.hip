@@ -26,8 +26,9 @@
 // Against the eight-wavefront kernel (prefill_varlen.hip) on 8 x 4096 tokens, 32 q / 8 kv heads, d 128: a tile
 // period of 2430 cycles for three wavefront-tiles per SIMD (63 % of the matrix pipe inside the loop, against
 // 58 %), but about 27 thousand cycles per workgroup outside the loop (the wait for Q, 5700 cycles of it at the
-// first barrier; the launch of a 768-thread workgroup; the wind-down), against 10 thousand: the two come out
-// even there (0.40 of the bf16 peak), this one ahead by 7 to 10 % on shorter sequences and at head size 64.
+// first barrier; the launch of a 768-thread workgroup; the wind-down), against 10 thousand.  With the two kernels
+// taking turns on a warm device this one is 1 % behind there and 2 to 8 % behind on shorter sequences; it is
+// therefore kept as a kernel that a caller can ask for (prefill_kernel = 4), not one the library picks.
 #include "prefill_common.h"
 
 // The global -> LDS copies set M0 inside inline asm and name it in their clobber lists; M0 is a register
@@ -340,9 +341,6 @@ __global__ __launch_bounds__(768) void prefill_varlen_r3_kernel(PrefillParams p)
     }
     l_run += psum;
   };
-  // Tiles entirely past the diagonal of every row of this wavefront are skipped.
-  auto skip_tile = [&](int j) { return (wave_row0 >= Lq) || (p.causal && j * XBN > wave_last_row + off); };
-
   // ---- prologue: tiles 0 to 3 ----
 #pragma unroll
   for (int t0 = 0; t0 < 4; t0++)
@@ -494,15 +492,12 @@ bool dispatch_r3(const PrefillParams &p, hipStream_t stream) {
 
 }  // namespace
 
-// Measured on MI355X (causal, 32 q / 8 kv heads): 16 x 1024 tokens 221 against 245 us, eight ragged sequences of
-// 37..3000 tokens 196 against 210 us, 8 x 4096 tokens at head size 64 722 against 776 us; even at 8 x 4096 tokens
-// and head size 128 (1.10 ms either way); behind on launches of a few hundred workgroups (2 x 2048 tokens 101
-// against 97 us, 4 sequences of 128..512 tokens with 32 kv heads 29 against 24 us).
-bool prefer_prefill_r3(const PrefillParams &p) {
-  if (p.G % 4 != 0 || p.d > 128 || p.win_left >= 0 || p.win_right > 0 || p.block_tables != nullptr) return false;
-  const int64_t n_wg = (int64_t)((p.max_q + 95) / 96) * p.batch * (p.Hq / 4);
-  return n_wg >= 768 && (p.max_q <= 3072 || p.d <= 64);
-}
+// Never the library's own choice: measured on MI355X with the two kernels taking turns on a warm device (causal,
+// 32 q / 8 kv heads, head size 128) the eight-wavefront kernel is ahead by 2 to 8 % from 64 x 512 to 8 x 3072 tokens
+// and by 1 % at 8 x 4096; at head size 64 this one is ahead by 0 to 2 %.  (Timed one after the other, whichever
+// kernel runs second looks 3 to 6 % better: the part raises its clock under matrix load for tens of milliseconds.)
+// The kernel stays selectable (prefill_kernel = 4) and tested.
+bool prefer_prefill_r3(const PrefillParams &) { return false; }
 
 bool launch_prefill_r3(const PrefillParams &p, int dtype, hipStream_t stream) {
   // causal or unmasked only; a tile's 32 rows are addressed with unsigned 32-bit byte offsets

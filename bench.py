@@ -649,6 +649,33 @@ def main() -> None:
             "frac": round(p.flops() / (qms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
             "kernel": "prefill_varlen_w8_kernel, block images copied global -> LDS (hipattn_mha_varlen_fwd_paged)"}
         del p, kc, vc
+        # The same number of tokens in sequences half as long, on the library's choice of kernel (eight
+        # wavefronts) and on the kernel that rotates three groups of four wavefronts through the matrix pipe;
+        # the two take turns, because whichever runs later finds the part at a higher clock.
+        p = W.config3(1.0, batch=16, L=2048).to(dev)
+        for _ in range(40):
+            prefill_step()
+        turns = {0: [], 4: []}
+        try:
+            for rnd in range(6):
+                for kern in ((0, 4) if rnd % 2 == 0 else (4, 0)):
+                    K.tuning_set("prefill_kernel", kern)
+                    prefill_step()
+                    prefill_step()
+                    turns[kern].append(sum(event_times_ms(prefill_step, 20, stream)) / 20)
+        finally:
+            K.tuning_set("prefill_kernel", 0)
+        sms, rms = statistics.median(turns[0]), statistics.median(turns[4])
+        line["prefill"]["rows_of_2048"] = {
+            "value": round(p.flops() / (sms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": round(sms, 4),
+            "frac": round(p.flops() / (sms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "config": {"workload": "varlen causal prefill: 16 x 2048 tokens, 32 q / 8 kv heads, d 128, bf16, N(0,1)",
+                       "algorithmic_flops_per_step": p.flops()},
+            "kernel": "prefill_varlen_w8_kernel (the library's choice), HIP events on the launch stream",
+            "three_group_kernel_forced": {
+                "kernel": "prefill_varlen_r3_kernel (prefill_kernel = 4)", "ms_per_step": round(rms, 4),
+                "value": round(p.flops() / (rms * 1e-3) / 1e12, 1), "unit": "TFLOP/s"}}
+        del p
 
     # ---- optional: the streaming helpers -------------------------------------------------------------
     if args.streaming:
