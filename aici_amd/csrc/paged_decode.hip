@@ -134,6 +134,58 @@ __device__ __forceinline__ void pair_load(const DecodeParams &p, const T *kbase,
   }
 }
 
+// The same 32 tokens from caches with 8- or 32-token blocks, into the same registers: the kernels think in
+// runs of 16 tokens ("blocks" below: what one MFMA tile of scores covers), and a pair of them is one
+// 32-token block of the cache (id i0; its two halves) or four 8-token blocks (ids i0..i3; a lane's token
+// says which one it reads).  Ids are clamped like those of pair_load: a pair's trailing ids may lie past
+// the context, where the table holds anything; the tokens read through them are masked by the caller.
+template <typename T, int HD, int BS>
+__device__ __forceinline__ void pair_load_bs(const DecodeParams &p, const T *kbase, const T *vbase, int64_t i0, int64_t i1,
+                                             int64_t i2, int64_t i3, PairRegs<HD> &r) {
+  static_assert(BS == 8 || BS == 16 || BS == 32, "block sizes of the reference's support matrix");
+  if constexpr (BS == 16) {
+    pair_load<T, HD>(p, kbase, vbase, i0, i1, r);
+  } else {
+    constexpr int NCH = HD / 8;
+    constexpr int NSTEP = (HD + 31) / 32;
+    constexpr int NDT = HD / 16;
+    const int lane = threadIdx.x & 63;
+    const int kg = lane >> 4;
+    const int col = lane & 15;
+    const int64_t last_block = p.num_blocks - 1;
+    auto clamp = [&](int64_t b) { return b < 0 ? (int64_t)0 : (b > last_block ? last_block : b); };
+    const T *ka, *kb, *va, *vb;  // this lane's row of K (token col) and run of V (tokens 4kg..4kg+3) in each half
+    if constexpr (BS == 32) {
+      const int64_t b = clamp(i0);
+      ka = kbase + b * p.k_block_stride + col * 8;
+      kb = ka + 16 * 8;
+      va = vbase + b * p.v_block_stride + kg * 4;
+      vb = va + 16;
+    } else {
+      const int64_t ba = clamp(i0), bb = clamp(i1), bc = clamp(i2), bd = clamp(i3);
+      ka = kbase + (col < 8 ? ba : bb) * p.k_block_stride + (col & 7) * 8;
+      kb = kbase + (col < 8 ? bc : bd) * p.k_block_stride + (col & 7) * 8;
+      va = vbase + (kg < 2 ? ba : bb) * p.v_block_stride + (kg & 1) * 4;
+      vb = vbase + (kg < 2 ? bc : bd) * p.v_block_stride + (kg & 1) * 4;
+    }
+#pragma unroll
+    for (int s = 0; s < NSTEP; s++) {
+      const int ch = 4 * s + kg;
+      r.kra[s] = u32x4_t{0u, 0u, 0u, 0u};
+      r.krb[s] = u32x4_t{0u, 0u, 0u, 0u};
+      if (NCH % 4 == 0 || ch < NCH) {
+        r.kra[s] = *reinterpret_cast<const u32x4_t *>(ka + ch * BS * 8);
+        r.krb[s] = *reinterpret_cast<const u32x4_t *>(kb + ch * BS * 8);
+      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++) {
+      r.vra[dt] = *reinterpret_cast<const u32x2_t *>(va + (dt * 16 + col) * BS);
+      r.vrb[dt] = *reinterpret_cast<const u32x2_t *>(vb + (dt * 16 + col) * BS);
+    }
+  }
+}
+
 // Folds a loaded block pair -- blocks `blk` and `blk + 1` of the context, the
 // second absent when !has_b -- into the running softmax state (m_run, l_run,
 // acc).  qreg: lane (kg, col) holds q[head col][32*step + 8*kg .. +8].
@@ -227,7 +279,8 @@ __device__ __forceinline__ void pair_step(const DecodeParams &p, const T *kbase,
 
 // V2FMT: write partials in the reference's v2 layout (normalised T outputs,
 // natural-log maxima) instead of the internal fp32 one.
-template <typename T, int HD, bool V2FMT>
+// BS: tokens per block of the cache; inside, a "block" is a run of 16 tokens whatever BS is.
+template <typename T, int HD, bool V2FMT, int BS>
 __global__ __launch_bounds__(256) void paged_decode_kernel(DecodeParams p) {
   typedef typename Vec8<T>::type vec8;
   constexpr int NCH = HD / 8;             // 16-byte chunks per K row
@@ -250,8 +303,12 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(DecodeParams p) {
   // before the context length is known (rows are zero-padded to max_blocks),
   // so the two round trips overlap.
   const int b0 = part * p.part_blocks;
+  const int t0 = b0 * kBlockSize / BS;            // the partition's first table column (b0 is even)
+  const int tn = p.part_blocks * kBlockSize / BS;  // and how many it has: at most 64, with 8-token blocks 128
   int tbl = 0;
-  if (lane < p.part_blocks && b0 + lane < p.table_cols) tbl = p.block_tables[seq * p.max_blocks + b0 + lane];
+  if (lane < tn && t0 + lane < p.table_cols) tbl = p.block_tables[seq * p.max_blocks + t0 + lane];
+  int tbl_hi = 0;
+  if (BS == 8 && 64 + lane < tn && t0 + 64 + lane < p.table_cols) tbl_hi = p.block_tables[seq * p.max_blocks + t0 + 64 + lane];
   const int ctx = min(p.context_lens[seq], p.max_ctx);
   const int nblk = (ctx + kBlockSize - 1) / kBlockSize;
   const int g_idx = cg * 16 + col;  // query head within the GQA group
@@ -298,9 +355,23 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(DecodeParams p) {
 
   for (int it = 2 * wave; it < nb; it += 8) {
     const bool has_b = it + 1 < nb;
-    const int64_t pa = __builtin_amdgcn_readlane(tbl, it);
-    const int64_t pb = __builtin_amdgcn_readlane(tbl, has_b ? it + 1 : it);
-    pair_step<T, HD>(p, kbase, vbase, pa, pb, b0 + it, has_b, ctx, slope, qreg, m_run, l_run, acc);
+    int64_t i0, i1 = 0, i2 = 0, i3 = 0;
+    if constexpr (BS == 16) {
+      i0 = __builtin_amdgcn_readlane(tbl, it);
+      i1 = __builtin_amdgcn_readlane(tbl, has_b ? it + 1 : it);
+    } else if constexpr (BS == 32) {
+      i0 = __builtin_amdgcn_readlane(tbl, it >> 1);
+    } else {
+      const int c = (2 * it) & 63;  // four columns that never straddle the two registers
+      const int src = 2 * it < 64 ? tbl : tbl_hi;
+      i0 = __builtin_amdgcn_readlane(src, c);
+      i1 = __builtin_amdgcn_readlane(src, c + 1);
+      i2 = __builtin_amdgcn_readlane(src, c + 2);
+      i3 = __builtin_amdgcn_readlane(src, c + 3);
+    }
+    PairRegs<HD> r;
+    pair_load_bs<T, HD, BS>(p, kbase, vbase, i0, i1, i2, i3, r);
+    pair_compute<T, HD>(p, r, b0 + it, has_b, ctx, slope, qreg, m_run, l_run, acc);
   }
 
   float l_tot = l_run + __shfl_xor(l_run, 16, 64);
@@ -429,12 +500,12 @@ __global__ __launch_bounds__(THREADS) void paged_decode_reduce_kernel(DecodePara
   }
 }
 
-template <typename T, int HD, bool V2FMT>
+template <typename T, int HD, bool V2FMT, int BS>
 void launch_decode(const DecodeParams &p, int64_t S, hipStream_t stream) {
   const int64_t n_wg = (int64_t)p.num_parts * p.Hkv * p.col_groups * S;
   HA_CHECK(n_wg <= 0x7fffffff, "paged_attention: too many workgroups");
   dim3 grid((unsigned)n_wg);
-  paged_decode_kernel<T, HD, V2FMT><<<grid, 256, 0, stream>>>(p);
+  paged_decode_kernel<T, HD, V2FMT, BS><<<grid, 256, 0, stream>>>(p);
   check_launch("paged_attention");
   if (p.num_parts > 1) {
     // few partitions: one slice of threads is enough and cheaper to start
@@ -447,17 +518,36 @@ void launch_decode(const DecodeParams &p, int64_t S, hipStream_t stream) {
   }
 }
 
-template <typename T, bool V2FMT>
+template <typename T, bool V2FMT, int BS>
 void dispatch_head(const DecodeParams &p, int head_size, int64_t S, hipStream_t stream) {
   switch (head_size) {
-    case 64: launch_decode<T, 64, V2FMT>(p, S, stream); break;
-    case 80: launch_decode<T, 80, V2FMT>(p, S, stream); break;
-    case 96: launch_decode<T, 96, V2FMT>(p, S, stream); break;
-    case 112: launch_decode<T, 112, V2FMT>(p, S, stream); break;
-    case 128: launch_decode<T, 128, V2FMT>(p, S, stream); break;
-    case 256: launch_decode<T, 256, V2FMT>(p, S, stream); break;
+    case 64: launch_decode<T, 64, V2FMT, BS>(p, S, stream); break;
+    case 80: launch_decode<T, 80, V2FMT, BS>(p, S, stream); break;
+    case 96: launch_decode<T, 96, V2FMT, BS>(p, S, stream); break;
+    case 112: launch_decode<T, 112, V2FMT, BS>(p, S, stream); break;
+    case 128: launch_decode<T, 128, V2FMT, BS>(p, S, stream); break;
+    case 256: launch_decode<T, 256, V2FMT, BS>(p, S, stream); break;
     default: fail("paged_attention: unsupported head size %d (supported: 64, 80, 96, 112, 128, 256)", head_size);
   }
+}
+
+template <typename T, bool V2FMT>
+void dispatch_block_size(const DecodeParams &p, int head_size, int block_size, int64_t S, hipStream_t stream) {
+  switch (block_size) {
+    case 8: dispatch_head<T, V2FMT, 8>(p, head_size, S, stream); break;
+    case 16: dispatch_head<T, V2FMT, 16>(p, head_size, S, stream); break;
+    case 32: dispatch_head<T, V2FMT, 32>(p, head_size, S, stream); break;
+    default: fail("paged_attention: unsupported block size %d (supported: 8, 16, 32)", block_size);
+  }
+}
+
+// The head sizes the MFMA kernels are built for (the reference's list, attention_kernels.cu:663-699).
+bool mfma_head_size(int d) { return d == 64 || d == 80 || d == 96 || d == 112 || d == 128 || d == 256; }
+
+// Which calls the plain fp32 kernel takes: fp32 caches, and 8- / 32-token blocks at head sizes outside
+// that list (which it serves for any multiple of x up to 256, the MFMA kernels do not).
+bool takes_generic_kernel(int dtype, int block_size, int head_size) {
+  return dtype == HIPATTN_F32 || (block_size != kBlockSize && !mfma_head_size(head_size));
 }
 
 // ---------------------------------------------------------------------------
@@ -867,7 +957,7 @@ int choose_part_blocks(int64_t S, int Hkv, int col_groups, int max_ctx) {
 
 DecodePlan plan_decode(int64_t S, int Hq, int Hkv, int head_size, int block_size, int dtype, int max_context_len) {
   DecodePlan pl;
-  pl.generic = block_size != kBlockSize || dtype == HIPATTN_F32;
+  pl.generic = takes_generic_kernel(dtype, block_size, head_size);
   if (S <= 0 || Hq <= 0) return pl;
   if (pl.generic) {
     int64_t P = ((int64_t)max_context_len + kGenericPartTokens - 1) / kGenericPartTokens;
@@ -877,7 +967,8 @@ DecodePlan plan_decode(int64_t S, int Hq, int Hkv, int head_size, int block_size
     if (P > 1) pl.slots = (size_t)S * Hq * P;
   } else {
     const int G = Hq / Hkv, col_groups = (G + 15) / 16;
-    pl.flat = use_flat_split(S, Hkv * col_groups, max_context_len);
+    // the flat split is built for 16-token blocks only (what rLLM runs); other block sizes take the partitioned launch
+    pl.flat = block_size == kBlockSize && use_flat_split(S, Hkv * col_groups, max_context_len);
     if (pl.flat) {
       const int64_t max_units = S * Hkv * col_groups * ((max_context_len + 2 * kBlockSize - 1) / (2 * kBlockSize));
       // What the device holds at once, but no more than gives every wavefront two units of the largest
@@ -1029,9 +1120,8 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
            "%s: block_tables and context_lens must be int32", op);
   HA_CHECK(block_size == 8 || block_size == 16 || block_size == 32,
            "%s: unsupported block size %d (supported: 8, 16, 32)", op, block_size);
-  // The MFMA kernels take 16-token blocks of a 2-byte type (what rLLM runs); the rest of the
-  // reference's support matrix goes to the fp32-FMA kernel.
-  const bool generic = block_size != kBlockSize || query->dtype == HIPATTN_F32;
+  // The MFMA kernels take the 2-byte types at the reference's head sizes; fp32 caches go to the fp32-FMA kernel.
+  const bool generic = takes_generic_kernel(query->dtype, block_size, (int)query->sizes[2]);
   const int x = 16 / dtype_size(query->dtype);
   const int64_t S = query->sizes[0];
   const int Hq = (int)query->sizes[1];
@@ -1115,7 +1205,6 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
   // A context length beyond max_context_len (which sized the launch and the scratch memory) or beyond
   // what a table row describes is cut there, in every kernel alike.
   p.max_ctx = (int)std::min<int64_t>(max_context_len, block_tables->sizes[1] * block_size);
-  const int64_t max_blocks = (max_context_len + block_size - 1) / block_size;
   if (v2) {
     check_tensor(exp_sums, "exp_sums", 3);
     check_tensor(max_logits, "max_logits", 3);
@@ -1144,7 +1233,9 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
       paged_decode_generic(g, query->dtype, true, max_context_len, (int)P, nullptr, stream);
       return;
     }
-    int64_t pb = (max_blocks + P - 1) / P;
+    // partition length in runs of 16 tokens, whatever the cache's block size
+    const int64_t max_runs = ((int64_t)max_context_len + kBlockSize - 1) / kBlockSize;
+    int64_t pb = (max_runs + P - 1) / P;
     if (pb < 2) pb = 2;
     pb += pb & 1;
     HA_CHECK(pb <= 64, "%s: %lld partitions are too few for max_context_len %d (at most 1024 tokens each)", op,
@@ -1177,9 +1268,9 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
       p.ws_l = p.ws_m + pl.slots;
     }
   }
-#define HA_PA(TT)                                          \
-  if (v2) dispatch_head<TT, true>(p, hd, S, stream);       \
-  else dispatch_head<TT, false>(p, hd, S, stream)
+#define HA_PA(TT)                                                          \
+  if (v2) dispatch_block_size<TT, true>(p, hd, block_size, S, stream);     \
+  else dispatch_block_size<TT, false>(p, hd, block_size, S, stream)
   if (query->dtype == HIPATTN_F16) {
     HA_PA(half_t);
   } else {

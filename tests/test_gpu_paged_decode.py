@@ -219,7 +219,8 @@ def test_argument_errors(device):
 
 
 # The rest of the reference's support matrix (attention_kernels.cu:594-700: block sizes 8/16/32,
-# float / half / bf16) runs on a plain fp32 kernel.
+# float / half / bf16): 8- and 32-token blocks of a 2-byte type run on the MFMA kernels (partitioned launch) at the
+# reference's head sizes, float caches and other head sizes on a plain fp32 kernel.
 FP32_TOL = 2e-5
 
 
@@ -287,6 +288,52 @@ def test_other_block_sizes_edges_alibi_and_stale_slots(device, dtype, bs):
     assert torch.equal(out[1].cpu(), one.to(dtype))
     tol = 5e-5 if dtype == torch.float32 else TOL[dtype]
     assert (out.cpu().float() - want).abs().max().item() <= tol
+
+
+@pytest.mark.parametrize("dtype,heads", [(torch.bfloat16, (32, 8, 128)), (torch.float16, (40, 1, 64)),
+                                         (torch.bfloat16, (8, 8, 80)), (torch.float16, (6, 2, 256))])
+@pytest.mark.parametrize("part_blocks", [0, 2, 64])
+def test_block_sizes_8_and_32_give_the_bits_of_block_size_16(device, tuning, dtype, heads, part_blocks):
+    """The MFMA kernels walk a context in runs of 16 tokens whatever the cache's block size is, so the same keys
+    and values scattered into caches of 8-, 16- and 32-token blocks (each with its own shuffled table, the
+    unused slots holding NaN) must give the same bits when the contexts are cut into the same partitions --
+    the library's own choice, the shortest (2 runs) and the longest (64 runs: with 8-token blocks a partition
+    then spans 128 table columns).  One of them is held against the float64 statement."""
+    Hq, Hkv, d = heads
+    tuning("decode_flat", 0)
+    tuning("decode_part_blocks", part_blocks)
+    lens = [1, 7, 17, 500, 1111, 2049, 4100]
+    S, T = len(lens), sum(lens)
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn((S, Hq, d), generator=g).to(dtype)
+    k = torch.randn((T, Hkv, d), generator=g).to(dtype)
+    v = torch.randn((T, Hkv, d), generator=g).to(dtype)
+    ctx = torch.tensor(lens, dtype=torch.int32)
+    outs = {}
+    for bs in (16, 8, 32):
+        nblk = [(l + bs - 1) // bs for l in lens]
+        pool = sum(nblk) + 7
+        perm = np.random.default_rng(bs).permutation(pool)
+        tables = np.zeros((S, max(nblk)), dtype=np.int32)
+        slots, pos = [], 0
+        for i, n in enumerate(nblk):
+            tables[i, :n] = perm[pos:pos + n]
+            slots += W.slots_for(perm[pos:pos + n].tolist(), lens[i], bs)
+            pos += n
+        kshape, vshape = W.cache_shapes(pool, Hkv, d, bs, dtype)
+        kc = torch.full(kshape, float("nan"), dtype=dtype, device=device)
+        vc = torch.full(vshape, float("nan"), dtype=dtype, device=device)
+        K.reshape_and_cache(k.to(device), v.to(device), kc, vc, torch.tensor(slots, dtype=torch.int64, device=device))
+        out = torch.full((S, Hq, d), float("nan"), dtype=dtype, device=device)
+        K.paged_attention_v1(out, q.to(device), kc, vc, Hkv, d ** -0.5, torch.from_numpy(tables).to(device),
+                             ctx.to(device), bs, max(lens))
+        outs[bs] = out.cpu()
+        assert not torch.isnan(outs[bs]).any()
+        if bs == 8:
+            want = ref.paged_attention_fp64(q, torch.nan_to_num(kc.cpu()), torch.nan_to_num(vc.cpu()), Hkv, d ** -0.5,
+                                            torch.from_numpy(tables), ctx, bs)
+            assert (outs[bs].double() - want).abs().max().item() <= TOL[dtype]
+    assert torch.equal(outs[8], outs[16]) and torch.equal(outs[32], outs[16])
 
 
 # ---- scratch memory: caller-provided workspaces, streams, context lengths beyond the stated maximum ----
