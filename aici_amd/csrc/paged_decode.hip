@@ -168,20 +168,27 @@ __device__ __forceinline__ void pair_load_bs(const DecodeParams &p, const T *kba
       va = vbase + (kg < 2 ? ba : bb) * p.v_block_stride + (kg & 1) * 4;
       vb = vbase + (kg < 2 ? bc : bd) * p.v_block_stride + (kg & 1) * 4;
     }
+    // A load instruction reaches 4 KiB either side of its address register.  With 32-token blocks the steps of
+    // a block lie 2 KiB apart and its tiles 1 KiB, so the lane addresses point 4 KiB into the block and the
+    // steps and tiles are reached by constants on both sides: one address register per operand, as with
+    // 16-token blocks (where everything lies within 4 KiB of the block's start).
+    constexpr int BIAS = BS == 32 ? 2048 : 0;  // elements
+    const T *kal = ka + kg * BS * 8 + BIAS, *kbl = kb + kg * BS * 8 + BIAS;
+    const T *val = va + col * BS + BIAS, *vbl = vb + col * BS + BIAS;
 #pragma unroll
     for (int s = 0; s < NSTEP; s++) {
       const int ch = 4 * s + kg;
       r.kra[s] = u32x4_t{0u, 0u, 0u, 0u};
       r.krb[s] = u32x4_t{0u, 0u, 0u, 0u};
       if (NCH % 4 == 0 || ch < NCH) {
-        r.kra[s] = *reinterpret_cast<const u32x4_t *>(ka + ch * BS * 8);
-        r.krb[s] = *reinterpret_cast<const u32x4_t *>(kb + ch * BS * 8);
+        r.kra[s] = *reinterpret_cast<const u32x4_t *>(kal + (4 * s * BS * 8 - BIAS));
+        r.krb[s] = *reinterpret_cast<const u32x4_t *>(kbl + (4 * s * BS * 8 - BIAS));
       }
     }
 #pragma unroll
     for (int dt = 0; dt < NDT; dt++) {
-      r.vra[dt] = *reinterpret_cast<const u32x2_t *>(va + (dt * 16 + col) * BS);
-      r.vrb[dt] = *reinterpret_cast<const u32x2_t *>(vb + (dt * 16 + col) * BS);
+      r.vra[dt] = *reinterpret_cast<const u32x2_t *>(val + (dt * 16 * BS - BIAS));
+      r.vrb[dt] = *reinterpret_cast<const u32x2_t *>(vbl + (dt * 16 * BS - BIAS));
     }
   }
 }
@@ -586,7 +593,7 @@ struct FlatSplit {
   }
 };
 
-template <typename T, int HD>
+template <typename T, int HD, int BS>
 __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void paged_decode_flat_kernel(DecodeParams p) {
   typedef typename Vec8<T>::type vec8;
   constexpr int NCH = HD / 8;
@@ -705,16 +712,29 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void paged_decode_flat_kern
     // The table entries of up to 32 pairs sit one per lane.
     for (int sp = 0; sp < n; sp += 32) {
       const int nsub = min(32, n - sp);
-      const int b_first = 2 * (pr0 + sp);
+      const int b_first = 2 * (pr0 + sp);             // in runs of 16 tokens
+      const int t_first = b_first * kBlockSize / BS;  // the table column of the first of them
       int tbl = 0;
-      if (b_first + lane < p.table_cols) tbl = p.block_tables[seq * p.max_blocks + b_first + lane];
+      if (lane < 64 * kBlockSize / BS && t_first + lane < p.table_cols)
+        tbl = p.block_tables[seq * p.max_blocks + t_first + lane];
+      int tbl_hi = 0;  // 8-token blocks: 32 pairs span 128 columns
+      if (BS == 8 && t_first + 64 + lane < p.table_cols) tbl_hi = p.block_tables[seq * p.max_blocks + t_first + 64 + lane];
       // Two register sets (heads up to 128 elements): the next pair's loads are
       // in flight while the current pair is folded in.
       auto issue = [&](int it, PairRegs<HD> &r) {
-        const bool has_b = b_first + 2 * it + 1 < nblk;
-        const int64_t pa = __builtin_amdgcn_readlane(tbl, 2 * it);
-        const int64_t pb = __builtin_amdgcn_readlane(tbl, has_b ? 2 * it + 1 : 2 * it);
-        pair_load<T, HD>(p, kbase, vbase, pa, pb, r);
+        if constexpr (BS == 16) {
+          const bool has_b = b_first + 2 * it + 1 < nblk;
+          const int64_t pa = __builtin_amdgcn_readlane(tbl, 2 * it);
+          const int64_t pb = __builtin_amdgcn_readlane(tbl, has_b ? 2 * it + 1 : 2 * it);
+          pair_load<T, HD>(p, kbase, vbase, pa, pb, r);
+        } else if constexpr (BS == 32) {
+          pair_load_bs<T, HD, BS>(p, kbase, vbase, __builtin_amdgcn_readlane(tbl, it), 0, 0, 0, r);
+        } else {
+          const int c = (4 * it) & 63;
+          const int src = it < 16 ? tbl : tbl_hi;
+          pair_load_bs<T, HD, BS>(p, kbase, vbase, __builtin_amdgcn_readlane(src, c), __builtin_amdgcn_readlane(src, c + 1),
+                                  __builtin_amdgcn_readlane(src, c + 2), __builtin_amdgcn_readlane(src, c + 3), r);
+        }
       };
       auto fold = [&](int it, PairRegs<HD> &r) {
         const int blk = b_first + 2 * it;
@@ -884,7 +904,7 @@ int flat_resident_workgroups() {
   if (r == 0) {
     int per_cu = 0, cus = 0;
     HA_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    HA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, paged_decode_flat_kernel<T, HD>, 256, 0));
+    HA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, paged_decode_flat_kernel<T, HD, kBlockSize>, 256, 0));
     r = (per_cu > 0 ? per_cu : 1) * (cus > 0 ? cus : 1);
     resident[dev].store(r, std::memory_order_relaxed);
   }
@@ -967,8 +987,7 @@ DecodePlan plan_decode(int64_t S, int Hq, int Hkv, int head_size, int block_size
     if (P > 1) pl.slots = (size_t)S * Hq * P;
   } else {
     const int G = Hq / Hkv, col_groups = (G + 15) / 16;
-    // the flat split is built for 16-token blocks only (what rLLM runs); other block sizes take the partitioned launch
-    pl.flat = block_size == kBlockSize && use_flat_split(S, Hkv * col_groups, max_context_len);
+    pl.flat = use_flat_split(S, Hkv * col_groups, max_context_len);
     if (pl.flat) {
       const int64_t max_units = S * Hkv * col_groups * ((max_context_len + 2 * kBlockSize - 1) / (2 * kBlockSize));
       // What the device holds at once, but no more than gives every wavefront two units of the largest
@@ -1045,28 +1064,34 @@ char *scratch_memory(const Scratch &from, const DecodePlan &pl, hipStream_t stre
 }
 
 template <typename T, int HD>
-void launch_decode_flat(DecodeParams p, const DecodePlan &pl, char *ws, hipStream_t stream) {
+void launch_decode_flat(DecodeParams p, const DecodePlan &pl, int block_size, char *ws, hipStream_t stream) {
   p.flat_waves = pl.flat_wgs * 4;
   p.flat_cols = pl.flat_cols;
   p.flat_prefix = reinterpret_cast<int *>(ws);
   p.ws_acc = reinterpret_cast<float *>(ws + pl.prefix_bytes);
   p.ws_m = p.ws_acc + pl.slots * HD;
   p.ws_l = p.ws_m + pl.slots;
-  paged_decode_flat_kernel<T, HD><<<dim3((unsigned)pl.flat_wgs), 256, 0, stream>>>(p);
+  // the three instances differ in their address arithmetic only: what the device holds of one it holds of all
+  switch (block_size) {
+    case 8: paged_decode_flat_kernel<T, HD, 8><<<dim3((unsigned)pl.flat_wgs), 256, 0, stream>>>(p); break;
+    case 32: paged_decode_flat_kernel<T, HD, 32><<<dim3((unsigned)pl.flat_wgs), 256, 0, stream>>>(p); break;
+    default: paged_decode_flat_kernel<T, HD, kBlockSize><<<dim3((unsigned)pl.flat_wgs), 256, 0, stream>>>(p); break;
+  }
   check_launch("paged_attention");
   paged_decode_flat_reduce_kernel<T, HD><<<dim3((unsigned)p.Hq, (unsigned)p.num_seqs), HD <= 64 ? 64 : 128, 0, stream>>>(p);
   check_launch("paged_attention reduce");
 }
 
 template <typename T>
-void dispatch_head_flat(const DecodeParams &p, int head_size, const DecodePlan &pl, char *ws, hipStream_t stream) {
+void dispatch_head_flat(const DecodeParams &p, int head_size, int block_size, const DecodePlan &pl, char *ws,
+                        hipStream_t stream) {
   switch (head_size) {
-    case 64: launch_decode_flat<T, 64>(p, pl, ws, stream); break;
-    case 80: launch_decode_flat<T, 80>(p, pl, ws, stream); break;
-    case 96: launch_decode_flat<T, 96>(p, pl, ws, stream); break;
-    case 112: launch_decode_flat<T, 112>(p, pl, ws, stream); break;
-    case 128: launch_decode_flat<T, 128>(p, pl, ws, stream); break;
-    case 256: launch_decode_flat<T, 256>(p, pl, ws, stream); break;
+    case 64: launch_decode_flat<T, 64>(p, pl, block_size, ws, stream); break;
+    case 80: launch_decode_flat<T, 80>(p, pl, block_size, ws, stream); break;
+    case 96: launch_decode_flat<T, 96>(p, pl, block_size, ws, stream); break;
+    case 112: launch_decode_flat<T, 112>(p, pl, block_size, ws, stream); break;
+    case 128: launch_decode_flat<T, 128>(p, pl, block_size, ws, stream); break;
+    case 256: launch_decode_flat<T, 256>(p, pl, block_size, ws, stream); break;
     default: fail("paged_attention: unsupported head size %d (supported: 64, 80, 96, 112, 128, 256)", head_size);
   }
 }
@@ -1255,9 +1280,9 @@ void paged_attention_impl(hipattn_tensor *out, hipattn_tensor *exp_sums, hipattn
     }
     if (pl.flat) {
       if (query->dtype == HIPATTN_F16)
-        dispatch_head_flat<half_t>(p, hd, pl, ws, stream);
+        dispatch_head_flat<half_t>(p, hd, block_size, pl, ws, stream);
       else
-        dispatch_head_flat<bf16_t>(p, hd, pl, ws, stream);
+        dispatch_head_flat<bf16_t>(p, hd, block_size, pl, ws, stream);
       return;
     }
     p.part_blocks = pl.part_blocks;

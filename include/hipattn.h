@@ -121,10 +121,9 @@ char *hipattn_mha_varlen_fwd_paged(const hipattn_tensor *q, const hipattn_tensor
  * shapes before capturing, or use hipattn_paged_attention_v1_ws.
  * x = 16 / sizeof(dtype).  The reference's support matrix is accepted: f16,
  * bf16 and f32; BS 8, 16 and 32; d in {64, 80, 96, 112, 128, 256}.  The
- * 2-byte types take the MFMA kernels at every block size (BS = 16, what rLLM
- * runs, with both launch strategies; 8 and 32 with the partitioned one); f32
- * caches, and BS 8 / 32 at other head sizes (any d <= 256 that is a multiple
- * of x), take a plain fp32 kernel. */
+ * 2-byte types take the MFMA kernels at every block size; f32 caches, and
+ * BS 8 / 32 at other head sizes (any d <= 256 that is a multiple of x), take
+ * a plain fp32 kernel. */
 char *hipattn_paged_attention_v1(hipattn_tensor *out,
                                  const hipattn_tensor *query,
                                  const hipattn_tensor *key_cache,

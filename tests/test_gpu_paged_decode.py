@@ -292,16 +292,19 @@ def test_other_block_sizes_edges_alibi_and_stale_slots(device, dtype, bs):
 
 @pytest.mark.parametrize("dtype,heads", [(torch.bfloat16, (32, 8, 128)), (torch.float16, (40, 1, 64)),
                                          (torch.bfloat16, (8, 8, 80)), (torch.float16, (6, 2, 256))])
-@pytest.mark.parametrize("part_blocks", [0, 2, 64])
+@pytest.mark.parametrize("part_blocks", [0, 2, 64, "flat"])
 def test_block_sizes_8_and_32_give_the_bits_of_block_size_16(device, tuning, dtype, heads, part_blocks):
     """The MFMA kernels walk a context in runs of 16 tokens whatever the cache's block size is, so the same keys
     and values scattered into caches of 8-, 16- and 32-token blocks (each with its own shuffled table, the
-    unused slots holding NaN) must give the same bits when the contexts are cut into the same partitions --
-    the library's own choice, the shortest (2 runs) and the longest (64 runs: with 8-token blocks a partition
-    then spans 128 table columns).  One of them is held against the float64 statement."""
+    unused slots holding NaN) must give the same bits when the contexts are cut in the same places -- partitions
+    of the library's own choice, the shortest (2 runs) and the longest (64 runs: with 8-token blocks a partition
+    then spans 128 table columns), and the flat split.  One of them is held against the float64 statement."""
     Hq, Hkv, d = heads
-    tuning("decode_flat", 0)
-    tuning("decode_part_blocks", part_blocks)
+    if part_blocks == "flat":          # one list of block pairs cut into equal ranges: the same cut at every block size
+        tuning("decode_flat", 1)
+    else:
+        tuning("decode_flat", 0)
+        tuning("decode_part_blocks", part_blocks)
     lens = [1, 7, 17, 500, 1111, 2049, 4100]
     S, T = len(lens), sum(lens)
     g = torch.Generator().manual_seed(77)
