@@ -195,6 +195,25 @@ def test_config2_full_size(device):
     assert got.float().abs().max().item() <= c.value_cache.float().abs().max().item()
 
 
+@pytest.mark.parametrize("bs", [8, 32])
+def test_config2_shape_at_the_other_block_sizes(device, bs):
+    """The decode configuration's full shape (64 sequences, contexts U[512, 4096], 32 q / 8 kv heads, d 128, bf16)
+    with the cache in 8- and 32-token blocks: all 64 sequences against the float64 statement."""
+    key = ("config2", bs)
+    if key not in _ORACLE_CACHE:
+        c = W.decode_inputs(2, 64, 512, 4096, 32, 8, 128, torch.bfloat16, 20000 * 16 // bs, block_size=bs)
+        _ORACLE_CACHE[key] = (c, ref.paged_attention_fp64(c.q, c.key_cache, c.value_cache, c.num_kv_heads, c.scale,
+                                                          c.block_tables, c.context_lens, bs))
+    c, want64 = _ORACLE_CACHE[key]
+    d = c.to(device)
+    out = torch.full_like(d.q, float("nan"))
+    K.paged_attention_v1(out, d.q, d.key_cache, d.value_cache, c.num_kv_heads, c.scale, d.block_tables, d.context_lens,
+                         bs, c.max_ctx)
+    got = out.cpu()
+    assert not torch.isnan(got).any()
+    assert (got.double() - want64).abs().max().item() <= TOL[torch.bfloat16]
+
+
 def test_argument_errors(device):
     c = W.decode_inputs(18, 2, 5, 40, 8, 2, 128, torch.float16, 16).to(device)
     out = torch.empty_like(c.q)
