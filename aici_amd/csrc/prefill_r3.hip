@@ -24,11 +24,11 @@
 // K.Q^T, O^T = V^T.P^T on v_mfma_f32_32x32x16) are those of the other prefill kernels (prefill_varlen.hip).
 //
 // Against the eight-wavefront kernel (prefill_varlen.hip) on 8 x 4096 tokens, 32 q / 8 kv heads, d 128: a tile
-// period of 2430 cycles for three wavefront-tiles per SIMD (63 % of the matrix pipe inside the loop, against
-// 58 %), but about 27 thousand cycles per workgroup outside the loop (the wait for Q, 5700 cycles of it at the
-// first barrier; the launch of a 768-thread workgroup; the wind-down), against 10 thousand.  With the two kernels
-// taking turns on a warm device this one is 1 % behind there and 2 to 8 % behind on shorter sequences; it is
-// therefore kept as a kernel that a caller can ask for (prefill_kernel = 4), not one the library picks.
+// period of 2400 to 2700 cycles for three 32-key wavefront-tiles per SIMD (57 to 63 % of the matrix pipe inside
+// the loop) against 3140 for two 64-key ones (65 %), and more cycles per workgroup outside the loop (the wait for
+// Q at the first barrier; the launch of a 768-thread workgroup; the wind-down).  With the two kernels taking
+// turns on a warm device this one is 1 % behind there and 2 to 8 % behind on shorter sequences; it is therefore
+// kept as a kernel that a caller can ask for (prefill_kernel = 4), not one the library picks.
 #include "prefill_common.h"
 
 // The global -> LDS copies set M0 inside inline asm and name it in their clobber lists; M0 is a register
