@@ -34,7 +34,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
 PROFILED = {
     "decode_traffic_bytes": 643.2e6,      # FETCH_SIZE + WRITE_SIZE per decode step, scaled by a 1 GiB copy
     "decode_traffic_source": "profiles/decode_c2_prefill_c3_hbm_traffic.md",
-    "decode_main_kernel_us": 116.8,       # paged_decode_flat_kernel, average duration in the kernel trace
+    "decode_main_kernel_us": 115.6,       # paged_decode_flat_kernel, average duration in the kernel trace
     "decode_reduce_kernel_us": 4.9,       # paged_decode_flat_reduce_kernel
     "decode_kernels_source": "profiles/decode_c2_prefill_c3_kernel_trace.md",
     "prefill_traffic_bytes": 706.5e6,     # FETCH_SIZE + WRITE_SIZE per prefill launch, same scaling
@@ -489,6 +489,9 @@ def main() -> None:
     ap.add_argument("--no-llama-step", action="store_true",
                     help="skip the full Llama-3-8B-shaped decode step with the AICI mask + greedy stage "
                          "(it allocates about 170 GB of HBM)")
+    ap.add_argument("--no-short-rows", action="store_true",
+                    help="drop the 16 x 2048-token prefill leg (two kernels in turns): keeps a kernel trace's prefill "
+                         "row to the headline configuration")
     ap.add_argument("--no-decode-c5-shape", action="store_true",
                     help="skip the decode attention of the full-model configuration at its own shape (one layer)")
     ap.add_argument("--mixed-step", action="store_true", help="(default; kept for old command lines)")
@@ -649,33 +652,34 @@ def main() -> None:
             "frac": round(p.flops() / (qms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
             "kernel": "prefill_varlen_w8_kernel, block images copied global -> LDS (hipattn_mha_varlen_fwd_paged)"}
         del p, kc, vc
-        # The same number of tokens in sequences half as long, on the library's choice of kernel (eight
-        # wavefronts) and on the kernel that rotates three groups of four wavefronts through the matrix pipe;
-        # the two take turns, because whichever runs later finds the part at a higher clock.
-        p = W.config3(1.0, batch=16, L=2048).to(dev)
-        for _ in range(40):
-            prefill_step()
-        turns = {0: [], 4: []}
-        try:
-            for rnd in range(6):
-                for kern in ((0, 4) if rnd % 2 == 0 else (4, 0)):
-                    K.tuning_set("prefill_kernel", kern)
-                    prefill_step()
-                    prefill_step()
-                    turns[kern].append(sum(event_times_ms(prefill_step, 20, stream)) / 20)
-        finally:
-            K.tuning_set("prefill_kernel", 0)
-        sms, rms = statistics.median(turns[0]), statistics.median(turns[4])
-        line["prefill"]["rows_of_2048"] = {
-            "value": round(p.flops() / (sms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": round(sms, 4),
-            "frac": round(p.flops() / (sms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-            "config": {"workload": "varlen causal prefill: 16 x 2048 tokens, 32 q / 8 kv heads, d 128, bf16, N(0,1)",
-                       "algorithmic_flops_per_step": p.flops()},
-            "kernel": "prefill_varlen_w8_kernel (the library's choice), HIP events on the launch stream",
-            "three_group_kernel_forced": {
-                "kernel": "prefill_varlen_r3_kernel (prefill_kernel = 4)", "ms_per_step": round(rms, 4),
-                "value": round(p.flops() / (rms * 1e-3) / 1e12, 1), "unit": "TFLOP/s"}}
-        del p
+        if not args.no_short_rows:
+            # The same number of tokens in sequences half as long, on the library's choice of kernel (eight
+            # wavefronts) and on the kernel that rotates three groups of four wavefronts through the matrix pipe;
+            # the two take turns, because whichever runs later finds the part at a higher clock.
+            p = W.config3(1.0, batch=16, L=2048).to(dev)
+            for _ in range(40):
+                prefill_step()
+            turns = {0: [], 4: []}
+            try:
+                for rnd in range(6):
+                    for kern in ((0, 4) if rnd % 2 == 0 else (4, 0)):
+                        K.tuning_set("prefill_kernel", kern)
+                        prefill_step()
+                        prefill_step()
+                        turns[kern].append(sum(event_times_ms(prefill_step, 20, stream)) / 20)
+            finally:
+                K.tuning_set("prefill_kernel", 0)
+            sms, rms = statistics.median(turns[0]), statistics.median(turns[4])
+            line["prefill"]["rows_of_2048"] = {
+                "value": round(p.flops() / (sms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "ms_per_step": round(sms, 4),
+                "frac": round(p.flops() / (sms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                "config": {"workload": "varlen causal prefill: 16 x 2048 tokens, 32 q / 8 kv heads, d 128, bf16, N(0,1)",
+                           "algorithmic_flops_per_step": p.flops()},
+                "kernel": "prefill_varlen_w8_kernel (the library's choice), HIP events on the launch stream",
+                "three_group_kernel_forced": {
+                    "kernel": "prefill_varlen_r3_kernel (prefill_kernel = 4)", "ms_per_step": round(rms, 4),
+                    "value": round(p.flops() / (rms * 1e-3) / 1e12, 1), "unit": "TFLOP/s"}}
+            del p
 
     # ---- optional: the streaming helpers -------------------------------------------------------------
     if args.streaming:
