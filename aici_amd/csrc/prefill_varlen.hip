@@ -166,6 +166,33 @@ __global__ __launch_bounds__(256) void prefill_varlen_kernel(PrefillParams p) {
       // (block r, chunk, token), V unit (block r, head element, half of the block's tokens).  Blocks past the
       // context re-read its last one (their keys are masked, their V runs cleared before they reach LDS).
       staged_k0 = k0;
+      if (p.block_log2 != 4) {
+        // Caches of 8- or 32-token blocks: the same units -- a 16-byte run of K is (chunk, token) and one of V
+        // (head element, 8 tokens) at any block size -- each finding its own block: the id comes from the
+        // table row per unit, and the block's pitch takes the place of the 16.
+        const int bl = p.block_log2, bs = 1 << bl;
+        const int last_col = max(min((Lk - 1) >> bl, p.table_cols - 1), 0);
+        auto block_of = [&](int pos) -> int64_t {
+          const int id = table_row[min(pos >> bl, last_col)];
+          return id < 0 ? 0 : (id >= p.num_blocks ? p.num_blocks - 1 : (int64_t)id);
+        };
+        constexpr int K_PER_16 = CPR * 16, V_PER_16 = HDP * 2;
+#pragma unroll
+        for (int i = 0; i < NLOAD; i++) {
+          const int u = tid + 256 * i;
+          {
+            const int r = u / K_PER_16, rem = u % K_PER_16;
+            const int ch = min(rem / 16, d_chunks - 1), pos = k0 + r * 16 + rem % 16;
+            kst[i] = *reinterpret_cast<const u32x4_t *>(kp + block_of(pos) * p.kc_block + ((ch << bl) + (pos & (bs - 1))) * 8);
+          }
+          {
+            const int r = u / V_PER_16, rem = u % V_PER_16;
+            const int drow = min(rem / 2, p.d - 1), pos = k0 + r * 16 + (rem % 2) * 8;
+            vst[i] = *reinterpret_cast<const u32x4_t *>(vp + block_of(pos) * p.vc_block + (drow << bl) + (pos & (bs - 1)));
+          }
+        }
+        return;
+      }
       const int last_col = max(min((Lk - 1) >> 4, p.table_cols - 1), 0);
       int64_t blk[4];
 #pragma unroll
@@ -1508,6 +1535,21 @@ void dispatch_paged(const PrefillParams &p, hipStream_t stream) {
   // untouched, the rest is staged through registers, which pads it.  The tuning switch paged_prefill_dma = 0
   // forces the staged form.
   const bool dma = p.vc_block % 8 == 0 && p.vc_head % 8 == 0 && tuning().paged_prefill_dma != 0;
+  if (p.block_log2 != 4) {
+    // 8- and 32-token blocks (rLLM runs 16): the four-wavefront kernel, whose staged tiles take any block size
+    switch (hdp) {
+      case 32: launch_prefill<T, 32, 1, true>(p, stream); break;
+      case 64: launch_prefill<T, 64, 1, true>(p, stream); break;
+      case 96: launch_prefill<T, 96, 1, true>(p, stream); break;
+      case 128: launch_prefill<T, 128, 1, true>(p, stream); break;
+      case 160: launch_prefill<T, 160, 1, true>(p, stream); break;
+      case 192: launch_prefill<T, 192, 1, true>(p, stream); break;
+      case 224: launch_prefill<T, 224, 1, true>(p, stream); break;
+      case 256: launch_prefill<T, 256, 1, true>(p, stream); break;
+      default: fail("mha_varlen_fwd_paged: head size %d not supported (at most 256)", p.d);
+    }
+    return;
+  }
 #define HA_W8P(H)                                                                  \
   if (dma && p.d == H) launch_prefill_w8<T, H, W8_PAGED_DMA>(p, stream);           \
   else if (dma && H >= 64) launch_prefill_w8<T, (H >= 64 ? H : 64), W8_PAGED_DMA_PART>(p, stream); \
@@ -1546,13 +1588,15 @@ void mha_varlen_fwd_paged_impl(const hipattn_tensor *q, const hipattn_tensor *ke
   HA_CHECK(key_cache->dtype == q->dtype && value_cache->dtype == q->dtype, "%s: caches must have q's dtype", op);
   const int Hkv = (int)key_cache->sizes[1];
   HA_CHECK(Hkv > 0 && Hq % Hkv == 0, "%s: %d query heads not divisible by %d kv heads", op, Hq, Hkv);
-  HA_CHECK(key_cache->sizes[2] * key_cache->sizes[4] == d && key_cache->sizes[3] == 16 && key_cache->sizes[4] == 8,
-           "%s: key_cache shape does not match [nb, %d, %d/8, 16, 8]", op, Hkv, d);
+  const int64_t bs = key_cache->sizes[3];  // the caches say what their block size is
+  HA_CHECK(bs == 8 || bs == 16 || bs == 32, "%s: unsupported block size %lld (supported: 8, 16, 32)", op, (long long)bs);
+  HA_CHECK(key_cache->sizes[2] * key_cache->sizes[4] == d && key_cache->sizes[4] == 8,
+           "%s: key_cache shape does not match [nb, %d, %d/8, block size, 8]", op, Hkv, d);
   HA_CHECK(value_cache->sizes[0] == key_cache->sizes[0] && value_cache->sizes[1] == Hkv &&
-               value_cache->sizes[2] == d && value_cache->sizes[3] == 16,
-           "%s: value_cache shape does not match [nb, %d, %d, 16]", op, Hkv, d);
-  HA_CHECK(key_cache->strides[4] == 1 && key_cache->strides[3] == 8 && key_cache->strides[2] == 128 &&
-               value_cache->strides[3] == 1 && value_cache->strides[2] == 16,
+               value_cache->sizes[2] == d && value_cache->sizes[3] == bs,
+           "%s: value_cache shape does not match [nb, %d, %d, %lld]", op, Hkv, d, (long long)bs);
+  HA_CHECK(key_cache->strides[4] == 1 && key_cache->strides[3] == 8 && key_cache->strides[2] == 8 * bs &&
+               value_cache->strides[3] == 1 && value_cache->strides[2] == bs,
            "%s: cache inner dims must be contiguous", op);
   HA_CHECK(key_cache->strides[0] % 8 == 0 && key_cache->strides[1] % 8 == 0 && value_cache->strides[0] % 4 == 0 &&
                value_cache->strides[1] % 4 == 0 && (reinterpret_cast<uintptr_t>(key_cache->data) & 15) == 0 &&
@@ -1573,7 +1617,7 @@ void mha_varlen_fwd_paged_impl(const hipattn_tensor *q, const hipattn_tensor *ke
   HA_CHECK(block_tables->sizes[1] <= 1 || block_tables->strides[1] == 1, "%s: block_tables rows must be contiguous", op);
   HA_CHECK(scale > 0.f, "%s: softmax_scale must be positive", op);
   HA_CHECK(max_q >= 0 && max_k >= 0, "%s: negative max_seqlen", op);
-  HA_CHECK((int64_t)(max_k + 15) / 16 <= block_tables->sizes[1], "%s: max_seqlen_k %d needs more than the %lld block-table columns",
+  HA_CHECK(((int64_t)max_k + bs - 1) / bs <= block_tables->sizes[1], "%s: max_seqlen_k %d needs more than the %lld block-table columns",
            op, max_k, (long long)block_tables->sizes[1]);
   if (lse) {
     check_tensor(lse, "softmax_lse", 3);
@@ -1625,6 +1669,7 @@ void mha_varlen_fwd_paged_impl(const hipattn_tensor *q, const hipattn_tensor *ke
   p.kc_head = key_cache->strides[1];
   p.vc_block = value_cache->strides[0];
   p.vc_head = value_cache->strides[1];
+  p.block_log2 = bs == 8 ? 3 : (bs == 16 ? 4 : 5);
   if (q->dtype == HIPATTN_F16) dispatch_paged<half_t>(p, stream);
   else dispatch_paged<bf16_t>(p, stream);
 }

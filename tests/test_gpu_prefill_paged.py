@@ -27,23 +27,23 @@ def tile_route(request, tuning):
     return request.param
 
 
-def paged_case(seed, seqs, Hq, Hkv, d, dtype, pool):
-    """seqs: (prior, new) token counts.  Every context's K/V (prior and new) is in the cache; every slot no
-    context covers holds NaN, as an uninitialised cache may."""
+def paged_case(seed, seqs, Hq, Hkv, d, dtype, pool, bs=16):
+    """seqs: (prior, new) token counts.  Every context's K/V (prior and new) is in the cache (blocks of bs
+    tokens); every slot no context covers holds NaN, as an uninitialised cache may."""
     g = torch.Generator().manual_seed(seed)
     rng = np.random.default_rng(seed)
-    kc, vc = make_cache(pool, Hkv, d, 16, dtype, fill=float("nan"))
+    kc, vc = make_cache(pool, Hkv, d, bs, dtype, fill=float("nan"))
     perm = rng.permutation(pool).tolist()
     lens_k = [a + b for a, b in seqs]
     lens_q = [b for _, b in seqs]
-    width = max((l + 15) // 16 for l in lens_k)
+    width = max((l + bs - 1) // bs for l in lens_k)
     tables = np.zeros((len(seqs), width), dtype=np.int32)
     slots_all = []
     for i, lk in enumerate(lens_k):
-        n = (lk + 15) // 16
+        n = (lk + bs - 1) // bs
         blocks = [perm.pop() for _ in range(n)]
         tables[i, :n] = blocks
-        slots = torch.tensor(W.slots_for(blocks, lk), dtype=torch.int64)
+        slots = torch.tensor(W.slots_for(blocks, lk, bs), dtype=torch.int64)
         slots_all.append(slots)
         k = torch.randn((lk, Hkv, d), generator=g).to(dtype)
         v = torch.randn((lk, Hkv, d), generator=g).to(dtype)
@@ -85,6 +85,30 @@ def test_matches_oracle(device, dtype, heads):
     want = oracle(c, Hq, Hkv, d)
     assert not torch.isnan(got).any()
     assert (got.float() - want).abs().max().item() <= TOL[dtype]
+
+
+@pytest.mark.parametrize("bs", [8, 32])
+@pytest.mark.parametrize("dtype,heads", [(torch.bfloat16, (32, 8, 128)), (torch.float16, (32, 32, 80)), (torch.bfloat16, (4, 2, 8)),
+                                         (torch.float16, (6, 1, 96)), (torch.bfloat16, (4, 4, 72)), (torch.float16, (4, 2, 160)),
+                                         (torch.bfloat16, (8, 2, 256))])
+def test_caches_of_8_and_32_token_blocks(device, bs, dtype, heads):
+    """The reference's gather route works at any block size of the cache (gather_cached_kv takes slots); so does
+    the paged prefill, on the kernel that stages its tiles through registers: the same sequences as above,
+    with prior contexts that end inside blocks, against the oracle."""
+    Hq, Hkv, d = heads
+    c = paged_case(33, SEQS, Hq, Hkv, d, dtype, 420 * 16 // bs + 8, bs=bs)
+    got, lse = run_paged(c, device, lse=True)
+    want = oracle(c, Hq, Hkv, d)
+    assert not torch.isnan(got).any()
+    assert (got.cpu().float() - want).abs().max().item() <= TOL[dtype]
+    # and the same bits as from a cache of 16-token blocks holding the same keys and values (the kernel sees the
+    # same tiles), when that one is staged through registers as well
+    c16 = paged_case(33, SEQS, Hq, Hkv, d, dtype, 420, bs=16)
+    assert torch.equal(c16["q"], c["q"])
+    if d > 128 or K.tuning_get("paged_prefill_dma") == 0:
+        got16 = run_paged(c16, device)
+        if d > 128:
+            assert torch.equal(got16, got)
 
 
 @pytest.mark.parametrize("slope", [6.0, 0.5, -6.0])
