@@ -17,10 +17,9 @@ pytestmark = pytest.mark.gpu
 
 
 def mixed_step(seed, chunk_priors, chunk_len, n_decode, ctx_lo, ctx_hi, Hq, Hkv, d, dtype, pool, fused_qkv, device,
-               paged_prefill=False):
+               paged_prefill=False, bs=16):
     rng = np.random.default_rng(seed)
     g = torch.Generator().manual_seed(seed)
-    bs = 16
     alloc = paged.BlockAllocator(bs, pool)
     builder = paged.BatchInfoBuilder(bs, 1 << 20, paged_attn_kernel_v=1)
     kc, vc = make_cache(pool, Hkv, d, bs, dtype, fill=float("nan"))  # uninitialised cache
@@ -60,7 +59,7 @@ def mixed_step(seed, chunk_priors, chunk_len, n_decode, ctx_lo, ctx_hi, Hq, Hkv,
     lens_k = (bi.seqlens_k[1:] - bi.seqlens_k[:-1]).tolist() + bi.paged_context_lens.tolist()
     gather = bi.gather_mapping.tolist()
     for r in range(bi.paged_context_lens.numel()):
-        gather += W.slots_for(bi.paged_block_tables[r].tolist(), int(bi.paged_context_lens[r]))
+        gather += W.slots_for(bi.paged_block_tables[r].tolist(), int(bi.paged_context_lens[r]), bs)
     gm = torch.tensor(gather, dtype=torch.int32)
     gk = torch.empty((len(gather), Hkv, d), dtype=dtype)
     gv = torch.empty_like(gk)
@@ -113,6 +112,19 @@ def test_paged_prefill_route(device, case):
     assert not torch.isnan(y.float()).any()
     assert (y.float() - want).abs().max().item() <= TOL[dtype]
     assert torch.equal(kc.view(torch.int16), kc_ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("bs", [8, 32])
+@pytest.mark.parametrize("paged_prefill", [False, True])
+def test_mixed_step_with_8_and_32_token_blocks(device, bs, paged_prefill):
+    """The whole composition -- scatter, gather or block tables, prefill rows, decode rows -- on caches of the
+    other two block sizes of the reference's matrix."""
+    y, want, (kc, vc, kc_ref, vc_ref), bi = mixed_step(35, [0, 17, 640], 200, 33, 1, 900, 32, 8, 128, torch.bfloat16,
+                                                       2048 * 16 // bs, False, device, paged_prefill=paged_prefill, bs=bs)
+    assert not torch.isnan(y.float()).any()
+    assert (y.float() - want).abs().max().item() <= TOL[torch.bfloat16]
+    assert torch.equal(kc.view(torch.int16), kc_ref.view(torch.int16))
+    assert torch.equal(vc.view(torch.int16), vc_ref.view(torch.int16))
 
 
 def test_all_prefill_and_all_decode_steps(device):
