@@ -9,32 +9,51 @@
 namespace {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
+// NT: loads and stores carry the non-temporal hint (data touched once: not kept in the caches).
+template <bool NT>
+__device__ __forceinline__ u32x4 ld(const u32x4 *p) {
+  if constexpr (NT) return __builtin_nontemporal_load(p);
+  return *p;
+}
+template <bool NT>
+__device__ __forceinline__ void st(u32x4 *p, u32x4 v) {
+  if constexpr (NT)
+    __builtin_nontemporal_store(v, p);
+  else
+    *p = v;
+}
+
 // Reads `n` 16-byte words once; the xor is stored only if it hits a value it cannot have by chance, so the
 // loads stay and no traffic is written.
+template <bool NT>
 __global__ __launch_bounds__(256) void read_kernel(const u32x4 *__restrict__ src, unsigned int *sink, int64_t n) {
   unsigned int acc = 0;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
-    const u32x4 v = src[i];
+    const u32x4 v = ld<NT>(src + i);
     acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
   }
   if (acc == 0x9e3779b9u && sink) sink[0] = acc;
 }
+template <bool NT>
 __global__ __launch_bounds__(256) void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, int64_t n) {
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) dst[i] = src[i];
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    st<NT>(dst + i, ld<NT>(src + i));
 }
+template <bool NT>
 __global__ __launch_bounds__(256) void fill_kernel(u32x4 *__restrict__ dst, int64_t n) {
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
-    dst[i] = u32x4{1u, 2u, 3u, 4u};
+    st<NT>(dst + i, u32x4{1u, 2u, 3u, 4u});
 }
 // One workgroup per entry of `chunks`: reads the chunk with that number, `words` 16-byte words long (256 for
 // the 4 KiB in which the paged caches are read: one block of one kv head at head size 128, 16-bit).
+template <bool NT>
 __global__ __launch_bounds__(256) void read_chunks_kernel(const u32x4 *__restrict__ src, const int32_t *__restrict__ chunks,
                                                            unsigned int *sink, int64_t n_chunks, int words) {
   unsigned int acc = 0;
   for (int64_t k = blockIdx.x; k < n_chunks; k += gridDim.x) {
     const u32x4 *c = src + (int64_t)chunks[k] * words;
     for (int i = threadIdx.x; i < words; i += 256) {
-      const u32x4 v = c[i];
+      const u32x4 v = ld<NT>(c + i);
       acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
     }
   }
@@ -43,8 +62,8 @@ __global__ __launch_bounds__(256) void read_chunks_kernel(const u32x4 *__restric
 }  // namespace
 
 // mode 0 reads src once (dst may be null), 1 copies src to dst, 2 fills dst, 3 reads the chunks of src that
-// chunks[0..n_chunks) number (each 0 <= chunks[k] < bytes / chunk_bytes; chunk_bytes a multiple of 4096).
-// Returns 0, a hipError_t, or -1 for bad arguments.
+// chunks[0..n_chunks) number (each 0 <= chunks[k] < bytes / chunk_bytes; chunk_bytes a multiple of 4096);
+// mode + 8: the same with non-temporal loads and stores.  Returns 0, a hipError_t, or -1 for bad arguments.
 extern "C" int membench_probe(int mode, void *dst, const void *src, int64_t bytes, const int32_t *chunks, int64_t n_chunks,
                               int chunk_bytes, void *stream_arg) {
   hipStream_t stream = static_cast<hipStream_t>(stream_arg);
@@ -52,24 +71,32 @@ extern "C" int membench_probe(int mode, void *dst, const void *src, int64_t byte
   const int64_t n = bytes / 16;
   if (n == 0) return 0;
   const unsigned grid = (unsigned)std::min<int64_t>((n + 255) / 256, 65536);
-  switch (mode) {
+  const bool nt = (mode & 8) != 0;
+  switch (mode & ~8) {
     case 0:
       if (!src) return -1;
-      read_kernel<<<grid, 256, 0, stream>>>(static_cast<const u32x4 *>(src), static_cast<unsigned int *>(dst), n);
+      if (nt) read_kernel<true><<<grid, 256, 0, stream>>>(static_cast<const u32x4 *>(src), static_cast<unsigned int *>(dst), n);
+      else read_kernel<false><<<grid, 256, 0, stream>>>(static_cast<const u32x4 *>(src), static_cast<unsigned int *>(dst), n);
       break;
     case 1:
       if (!src || !dst) return -1;
-      copy_kernel<<<grid, 256, 0, stream>>>(static_cast<const u32x4 *>(src), static_cast<u32x4 *>(dst), n);
+      if (nt) copy_kernel<true><<<grid, 256, 0, stream>>>(static_cast<const u32x4 *>(src), static_cast<u32x4 *>(dst), n);
+      else copy_kernel<false><<<grid, 256, 0, stream>>>(static_cast<const u32x4 *>(src), static_cast<u32x4 *>(dst), n);
       break;
     case 2:
       if (!dst) return -1;
-      fill_kernel<<<grid, 256, 0, stream>>>(static_cast<u32x4 *>(dst), n);
+      if (nt) fill_kernel<true><<<grid, 256, 0, stream>>>(static_cast<u32x4 *>(dst), n);
+      else fill_kernel<false><<<grid, 256, 0, stream>>>(static_cast<u32x4 *>(dst), n);
       break;
     case 3: {
       if (!src || !chunks || n_chunks <= 0 || chunk_bytes <= 0 || chunk_bytes % 4096 != 0 || bytes % chunk_bytes != 0) return -1;
       const unsigned g = (unsigned)std::min<int64_t>(n_chunks, 16384);
-      read_chunks_kernel<<<g, 256, 0, stream>>>(static_cast<const u32x4 *>(src), chunks, static_cast<unsigned int *>(dst), n_chunks,
-                                                chunk_bytes / 16);
+      if (nt)
+        read_chunks_kernel<true><<<g, 256, 0, stream>>>(static_cast<const u32x4 *>(src), chunks, static_cast<unsigned int *>(dst),
+                                                        n_chunks, chunk_bytes / 16);
+      else
+        read_chunks_kernel<false><<<g, 256, 0, stream>>>(static_cast<const u32x4 *>(src), chunks, static_cast<unsigned int *>(dst),
+                                                         n_chunks, chunk_bytes / 16);
       break;
     }
     default: return -1;

@@ -90,6 +90,14 @@ struct Mfma16<bf16_t> {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// A load of cache bytes.  Every byte of K and V is read once per launch and never again: the loads carry the
+// non-temporal hint, so the lines are not kept in L2 and the memory-side cache at the expense of each other.
+// Measured on MI355X, 64 sequences of 512..4096 tokens, 8 kv heads x 128: 120.8 -> 107.2 us per step.
+template <typename V>
+__device__ __forceinline__ V stream_load(const V *p) {
+  return __builtin_nontemporal_load(p);
+}
+
 // The cache bytes of one block pair of one kv head, as MFMA operands.
 template <int HD>
 struct PairRegs {
@@ -121,16 +129,16 @@ __device__ __forceinline__ void pair_load(const DecodeParams &p, const T *kbase,
     r.kra[s] = u32x4_t{0u, 0u, 0u, 0u};
     r.krb[s] = u32x4_t{0u, 0u, 0u, 0u};
     if (NCH % 4 == 0 || ch < NCH) {
-      r.kra[s] = *reinterpret_cast<const u32x4_t *>(ka + (ch * kBlockSize + col) * 8);
-      r.krb[s] = *reinterpret_cast<const u32x4_t *>(kb + (ch * kBlockSize + col) * 8);
+      r.kra[s] = stream_load(reinterpret_cast<const u32x4_t *>(ka + (ch * kBlockSize + col) * 8));
+      r.krb[s] = stream_load(reinterpret_cast<const u32x4_t *>(kb + (ch * kBlockSize + col) * 8));
     }
   }
   // V: tile dt of a block is the contiguous 512 B run of rows 16dt..16dt+15;
   // lane (kg, row) takes tokens 4kg..4kg+3 of its row.
 #pragma unroll
   for (int dt = 0; dt < NDT; dt++) {
-    r.vra[dt] = *reinterpret_cast<const u32x2_t *>(va + (dt * 16 + col) * kBlockSize + kg * 4);
-    r.vrb[dt] = *reinterpret_cast<const u32x2_t *>(vb + (dt * 16 + col) * kBlockSize + kg * 4);
+    r.vra[dt] = stream_load(reinterpret_cast<const u32x2_t *>(va + (dt * 16 + col) * kBlockSize + kg * 4));
+    r.vrb[dt] = stream_load(reinterpret_cast<const u32x2_t *>(vb + (dt * 16 + col) * kBlockSize + kg * 4));
   }
 }
 
@@ -181,14 +189,14 @@ __device__ __forceinline__ void pair_load_bs(const DecodeParams &p, const T *kba
       r.kra[s] = u32x4_t{0u, 0u, 0u, 0u};
       r.krb[s] = u32x4_t{0u, 0u, 0u, 0u};
       if (NCH % 4 == 0 || ch < NCH) {
-        r.kra[s] = *reinterpret_cast<const u32x4_t *>(kal + (4 * s * BS * 8 - BIAS));
-        r.krb[s] = *reinterpret_cast<const u32x4_t *>(kbl + (4 * s * BS * 8 - BIAS));
+        r.kra[s] = stream_load(reinterpret_cast<const u32x4_t *>(kal + (4 * s * BS * 8 - BIAS)));
+        r.krb[s] = stream_load(reinterpret_cast<const u32x4_t *>(kbl + (4 * s * BS * 8 - BIAS)));
       }
     }
 #pragma unroll
     for (int dt = 0; dt < NDT; dt++) {
-      r.vra[dt] = *reinterpret_cast<const u32x2_t *>(val + (dt * 16 * BS - BIAS));
-      r.vrb[dt] = *reinterpret_cast<const u32x2_t *>(vbl + (dt * 16 * BS - BIAS));
+      r.vra[dt] = stream_load(reinterpret_cast<const u32x2_t *>(val + (dt * 16 * BS - BIAS)));
+      r.vrb[dt] = stream_load(reinterpret_cast<const u32x2_t *>(vbl + (dt * 16 * BS - BIAS)));
     }
   }
 }

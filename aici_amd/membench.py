@@ -26,13 +26,14 @@ def _load():
 
 
 def probe(mode: str, dst: Optional[torch.Tensor], src: Optional[torch.Tensor], chunks: Optional[torch.Tensor] = None,
-          chunk_bytes: int = 4096) -> None:
+          chunk_bytes: int = 4096, nontemporal: bool = False) -> None:
     """One launch on torch's current stream: "read" src once, "copy" src to dst, "fill" dst, or "read_chunks":
-    the chunks of src (chunk_bytes each) that the int32 tensor `chunks` numbers."""
+    the chunks of src (chunk_bytes each) that the int32 tensor `chunks` numbers; `nontemporal`: with the
+    hint on every load and store that the data is touched once."""
     modes = {"read": 0, "copy": 1, "fill": 2, "read_chunks": 3}
     t = src if src is not None else dst
     nbytes = t.numel() * t.element_size()
-    rc = _load().membench_probe(modes[mode], dst.data_ptr() if dst is not None else None,
+    rc = _load().membench_probe(modes[mode] + (8 if nontemporal else 0), dst.data_ptr() if dst is not None else None,
                                 src.data_ptr() if src is not None else None, nbytes,
                                 chunks.data_ptr() if chunks is not None else None,
                                 chunks.numel() if chunks is not None else 0, int(chunk_bytes),

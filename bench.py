@@ -195,6 +195,12 @@ def memory_system_leg(dev, stream, steps: int) -> dict:
     run("copy_1GiB_read_plus_write", lambda: membench.probe("copy", dst, src), 2 * n)
     run("fill_1GiB", lambda: membench.probe("fill", dst, None), n)
     run("read_4KiB_chunks_shuffled", lambda: membench.probe("read_chunks", None, big, order), order.numel() * 4096)
+    # the same with the non-temporal hint on every load and store (what the decode kernels' cache loads carry)
+    run("read_1GiB_nontemporal", lambda: membench.probe("read", None, src, nontemporal=True), n)
+    run("copy_1GiB_read_plus_write_nontemporal", lambda: membench.probe("copy", dst, src, nontemporal=True), 2 * n)
+    run("fill_1GiB_nontemporal", lambda: membench.probe("fill", dst, None, nontemporal=True), n)
+    run("read_4KiB_chunks_shuffled_nontemporal",
+        lambda: membench.probe("read_chunks", None, big, order, nontemporal=True), order.numel() * 4096)
     # the same amount in larger granules: what reading several kv heads of a block as one piece could give
     for kib in (16, 32):
         cb = kib * 1024
