@@ -302,11 +302,10 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
         for (int i = 0; i < 2; i++) {
           const int c = 4 * i + c4;
           if (c < nc)
-            *reinterpret_cast<uint4 *>(ks + tok * KP + c * X) =
-                *reinterpret_cast<const uint4 *>(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X);
+            *reinterpret_cast<uint4 *>(ks + tok * KP + c * X) = load16_once(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X);
           const int e = 32 * i + (lane >> 1);
           if (e < nc * X) {
-            const uint4 vin = *reinterpret_cast<const uint4 *>(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th);
+            const uint4 vin = load16_once(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th);
             const E *ve = reinterpret_cast<const E *>(&vin);
 #pragma unroll
             for (int t = 0; t < 8; t++) vs[(8 * th + t) * VP + e] = ve[t];
@@ -361,8 +360,8 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
         }
       } else {
         if (hi < nc) {
-          *reinterpret_cast<uint4 *>(ks + lo * KP + hi * X) = *reinterpret_cast<const uint4 *>(k_cache);
-          const uint4 vin = *reinterpret_cast<const uint4 *>(v_cache);
+          *reinterpret_cast<uint4 *>(ks + lo * KP + hi * X) = load16_once(k_cache);
+          const uint4 vin = load16_once(v_cache);
           const E *ve = reinterpret_cast<const E *>(&vin);
 #pragma unroll
           for (int t = 0; t < 8; t++) vs[t * VP + lane] = ve[t];

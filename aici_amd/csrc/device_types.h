@@ -60,6 +60,22 @@ __device__ __forceinline__ T sub_t(T a, T b) {
   return from_float<T>(to_float(a) - to_float(b));
 }
 
+// A 16-byte load of data that a kernel reads once: with the non-temporal hint the line is not kept in the
+// caches at the expense of data that is used again (or, in a purely streaming kernel, of the lines still on
+// their way).  HA_NT_STREAM = 0 builds the plain load, for comparison.
+#ifndef HA_NT_STREAM
+#define HA_NT_STREAM 1
+#endif
+__device__ __forceinline__ uint4 load16_once(const void *p) {
+#if HA_NT_STREAM
+  typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+  const v4u v = __builtin_nontemporal_load(static_cast<const v4u *>(p));
+  return make_uint4(v[0], v[1], v[2], v[3]);
+#else
+  return *static_cast<const uint4 *>(p);
+#endif
+}
+
 // Bit-pattern helpers for building MFMA operands out of 32-bit registers.
 template <typename V, typename U>
 __device__ __forceinline__ V bit_cast(const U &u) {

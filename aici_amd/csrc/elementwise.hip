@@ -90,8 +90,8 @@ __global__ __launch_bounds__(512) void rotary_neox_vec8_kernel(const Pos *__rest
     const int r = (i % per_head) * 8;
     T *arr = hd < num_heads ? query + token * q_stride + (int64_t)hd * head_size
                             : key + token * k_stride + (int64_t)(hd - num_heads) * head_size;
-    const uint4 xr = *reinterpret_cast<const uint4 *>(arr + r);
-    const uint4 yr = *reinterpret_cast<const uint4 *>(arr + embed + r);
+    const uint4 xr = load16_once(arr + r);
+    const uint4 yr = load16_once(arr + embed + r);
     const uint4 cr = *reinterpret_cast<const uint4 *>(cos_ptr + r);
     const uint4 sr = *reinterpret_cast<const uint4 *>(cos_ptr + embed + r);
     const T *x = reinterpret_cast<const T *>(&xr), *y = reinterpret_cast<const T *>(&yr);
@@ -157,7 +157,9 @@ __global__ __launch_bounds__(1024) void rms_norm_vec8_kernel(T *__restrict__ out
   float v[8];
   float ss = 0.f;
   if (active) {
-    const uint4 raw = *reinterpret_cast<const uint4 *>(x);
+    // (read-once hint only where the row is not written back in place: with the residual update it measured
+    // 2 % slower, without it 6 % faster, 32768 x 4096)
+    const uint4 raw = FUSED_ADD ? *reinterpret_cast<const uint4 *>(x) : load16_once(x);
     const T *e = reinterpret_cast<const T *>(&raw);
 #pragma unroll
     for (int j = 0; j < 8; j++) v[j] = to_float(e[j]);
@@ -224,8 +226,8 @@ __global__ __launch_bounds__(256) void silu_and_mul_vec8_kernel(T *__restrict__ 
   const int64_t row = blockIdx.y;
   const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (i >= d) return;
-  const uint4 xr = *reinterpret_cast<const uint4 *>(in + row * 2 * d + i);
-  const uint4 yr = *reinterpret_cast<const uint4 *>(in + row * 2 * d + d + i);
+  const uint4 xr = load16_once(in + row * 2 * d + i);
+  const uint4 yr = load16_once(in + row * 2 * d + d + i);
   const T *xe = reinterpret_cast<const T *>(&xr);
   const T *ye = reinterpret_cast<const T *>(&yr);
   uint4 o;
