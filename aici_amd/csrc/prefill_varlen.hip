@@ -567,7 +567,11 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
         const int r = idx / CPRQ, ch = idx % CPRQ;
         const int row = min(wave_row0 + r, Lq - 1);
         qraw[it] = u32x4_t{0u, 0u, 0u, 0u};
-        if (ch < d_chunks) qraw[it] = *reinterpret_cast<const u32x4_t *>(qp + (int64_t)row * p.q_row + ch * 8);
+        // (Q is read once and the output written once: with the non-temporal hint they do not displace the
+        // K / V tiles that the other row blocks of the sequence are about to fetch from L2 -- 8 x 4096 tokens
+        // 1.066 -> 1.051 ms from rows, 1.040 -> 1.019 ms from the paged cache; 16 x 1024 tokens 193 -> 188 us)
+        if (ch < d_chunks)
+          qraw[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(qp + (int64_t)row * p.q_row + ch * 8));
       }
     } else {
       const int row = min(wave_row0 + c, Lq - 1);
@@ -1307,8 +1311,8 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
     const int r = idx / CPRO, ch = idx % CPRO;
     const int row = wave_row0_e + r;
     if (((32 * CPRO) % 64 == 0 || r < 32) && row < Lq && ch < d_chunks)
-      *reinterpret_cast<u32x4_t *>(op + (int64_t)row * p.o_row + ch * 8) =
-          *reinterpret_cast<const u32x4_t *>(ost + r * OSTR + ch * 8);
+      __builtin_nontemporal_store(*reinterpret_cast<const u32x4_t *>(ost + r * OSTR + ch * 8),
+                                  reinterpret_cast<u32x4_t *>(op + (int64_t)row * p.o_row + ch * 8));
   }
   if (p.lse != nullptr && g_e == 0 && wave_row0_e + c_e < Lq) {
     const float lse = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : INFINITY;
