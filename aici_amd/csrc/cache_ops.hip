@@ -285,8 +285,9 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
         for (int i = 0; i < 2; i++) {  // chunk rows 4i + c4: 4 rows x 256 bytes per instruction
           const int c = 4 * i + c4;
           if (c < nc)
-            *reinterpret_cast<uint4 *>(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X) =
-                *reinterpret_cast<const uint4 *>(ks + tok * KP + c * X);
+            // (the cache is not read again before a later step: stored with the written-once hint, 47.8 -> 44.1 us
+            // for 32768 tokens x 8 kv heads x 128)
+            store16_once(kc_base + ((int64_t)(cg * 8 + c) * 16 + tok) * X, *reinterpret_cast<const uint4 *>(ks + tok * KP + c * X));
         }
 #pragma unroll
         for (int i = 0; i < 2; i++) {  // head elements 32i + lane / 2: 32 rows x 32 bytes per instruction
@@ -295,7 +296,7 @@ __global__ __launch_bounds__(256) void cache_move_tile_kernel(
           E *oe = reinterpret_cast<E *>(&o);
 #pragma unroll
           for (int t = 0; t < 8; t++) oe[t] = vs[(8 * th + t) * VP + e];
-          if (e < nc * X) *reinterpret_cast<uint4 *>(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th) = o;
+          if (e < nc * X) store16_once(vc_base + (int64_t)(cg * 64 + e) * 16 + 8 * th, o);
         }
       } else {
 #pragma unroll

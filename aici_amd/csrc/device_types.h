@@ -76,6 +76,17 @@ __device__ __forceinline__ uint4 load16_once(const void *p) {
 #endif
 }
 
+// The 16-byte store to match: data that nothing reads again soon.
+__device__ __forceinline__ void store16_once(void *p, uint4 v) {
+#if HA_NT_STREAM
+  typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+  v4u w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, static_cast<v4u *>(p));
+#else
+  *static_cast<uint4 *>(p) = v;
+#endif
+}
+
 // Bit-pattern helpers for building MFMA operands out of 32-bit registers.
 template <typename V, typename U>
 __device__ __forceinline__ V bit_cast(const U &u) {
