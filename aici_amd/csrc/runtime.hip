@@ -66,6 +66,9 @@ Tuning tuning_from_env() {
   t.prefill_wg_heads = env_int("HIPATTN_PREFILL_WG_HEADS", 0);
   t.prefill_rescale_log2 = env_int("HIPATTN_PREFILL_RESCALE_LOG2", 8);
   if (t.prefill_rescale_log2 < 0 || t.prefill_rescale_log2 > 16) t.prefill_rescale_log2 = 8;
+  t.linear_tiles = env_int("HIPATTN_LINEAR_TILES", 0);
+  t.linear_waves = env_int("HIPATTN_LINEAR_WAVES", 0);
+  t.linear_splits = env_int("HIPATTN_LINEAR_SPLITS", 0);
   return t;
 }
 Tuning g_tuning = tuning_from_env();  // once, when the library is loaded
@@ -84,6 +87,9 @@ const TuningField kTuningFields[] = {
     {"cache_move_lds", &Tuning::cache_move_lds, -1, 1},
     {"prefill_wg_heads", &Tuning::prefill_wg_heads, 0, 8},
     {"prefill_rescale_log2", &Tuning::prefill_rescale_log2, 0, 16},
+    {"linear_tiles", &Tuning::linear_tiles, 0, 2},
+    {"linear_waves", &Tuning::linear_waves, 0, 8},
+    {"linear_splits", &Tuning::linear_splits, 0, 32},
 };
 }  // namespace
 

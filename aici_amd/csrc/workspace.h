@@ -8,7 +8,7 @@
 namespace hipattn {
 
 // Which op a library-owned scratch buffer belongs to: ops never share one.
-enum WorkspaceUser { WS_PAGED_ATTENTION = 0, WS_BIAS_ARGMAX = 1 };
+enum WorkspaceUser { WS_PAGED_ATTENTION = 0, WS_BIAS_ARGMAX = 1, WS_LINEAR = 2 };
 
 // Returns at least `bytes` of device memory on the current device for `user`,
 // private to `stream`: calls on different streams never share a buffer, so
@@ -32,6 +32,9 @@ struct Tuning {
   int cache_move_lds;      // -1: the library chooses; 0: never the LDS-transposing kernels
   int prefill_wg_heads;      // eight-wavefront prefill: query heads of one kv group per workgroup, at most (0 and 1: one)
   int prefill_rescale_log2;  // prefill: a row's reference maximum moves when outgrown by more than 2^this (0..16, default 8)
+  int linear_tiles;          // linear: 16-row tiles of the weight per wavefront (0: the library chooses; 1 or 2)
+  int linear_waves;          // linear: wavefronts per workgroup (0: the library chooses; 4 or 8)
+  int linear_splits;         // linear: ranges of the inner dimension (0: the library chooses; else 1..32)
 };
 const Tuning &tuning();
 

@@ -246,6 +246,34 @@ def fused_add_rms_norm(input: torch.Tensor, residual: torch.Tensor, weight: torc
          float(epsilon), _stream(input))
 
 
+LINEAR_MAX_ROWS = 128
+
+
+def linear_takes(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether `linear` accepts these operands (else a caller multiplies with a library GEMM)."""
+    return (x.dim() == 2 and weight.dim() == 2 and 0 < x.size(0) <= LINEAR_MAX_ROWS and x.size(1) % 256 == 0
+            and weight.size(0) % 16 == 0 and x.dtype in (torch.float16, torch.bfloat16) and weight.dtype == x.dtype
+            and x.stride(1) == 1 and weight.stride(1) == 1 and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0)
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+           residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+           workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = x @ weight.T (+ bias) (+ residual) for at most 128 rows of x: `nn::Linear::forward` as rLLM calls
+    it for the rows of a generation step (llm/mod.rs:401-416; llama.rs:81-83, 96, 135-143, 210)."""
+    if out is None:
+        out = torch.empty((x.size(0), weight.size(0)), dtype=x.dtype, device=x.device)
+    call("hipattn_linear", _desc(out, "out"), _desc(x, "x"), _desc(weight, "weight"), _desc(bias, "bias"),
+         _desc(residual, "residual"), _desc(workspace, "workspace"), _stream(x))
+    return out
+
+
+def linear_workspace_size(x: torch.Tensor, weight: torch.Tensor) -> int:
+    n = ctypes.c_int64(0)
+    call("hipattn_linear_workspace_size", _desc(x, "x"), _desc(weight, "weight"), ctypes.byref(n))
+    return int(n.value)
+
+
 def silu_and_mul(out: torch.Tensor, input: torch.Tensor) -> None:
     call("hipattn_silu_and_mul", _desc(out, "out"), _desc(input, "input"), _stream(input))
 

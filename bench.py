@@ -394,7 +394,9 @@ def llama_step_leg(dev, stream, steps: int, layers: int, share_cache: bool) -> d
     """One full engine step of a Llama-3-8B-shaped model (random weights): 128 sequences decoding
     one token each over contexts U[1024,16384] (seed 5), every layer with its own paged KV cache,
     then the AICI step (5 % of the vocabulary allowed per sequence, packed bit masks) and greedy
-    arg-max.  Projections are library GEMMs; everything else runs through the C ABI."""
+    arg-max.  q/k/v, gate/up and lm_head are library GEMMs; o_proj and down_proj (few rows of the weight: a
+    library GEMM leaves most of the device idle) and everything else run through the C ABI.
+    `ms_per_step_library_gemms_only` is the same step with those two projections as library GEMMs as well."""
     import numpy as np
     import torch
 
@@ -439,6 +441,13 @@ def llama_step_leg(dev, stream, steps: int, layers: int, share_cache: bool) -> d
     same = bool(torch.equal(toks, step(False)))
     ms_ref = event_times_ms(lambda: step(False), steps, stream)
     ms_ref = sum(ms_ref) / len(ms_ref)
+    model.skinny_linear = False
+    # different summation orders, random weights: near-ties may fall the other way, so a count, not a check
+    equal_lib = int((toks == step()).sum())
+    ms_lib = event_times_ms(step, steps, stream)
+    ms_lib = sum(ms_lib) / len(ms_lib)
+    model.skinny_linear = True
+    step()
     ms = event_times_ms(step, steps, stream)
     ms = sum(ms) / len(ms)
     # the same step captured once in a HIP graph and replayed: no launch gaps between its ~400 kernels
@@ -471,6 +480,7 @@ def llama_step_leg(dev, stream, steps: int, layers: int, share_cache: bool) -> d
             "frac_of_hbm_peak": round((kv_bytes + weight_bytes) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "constrained_tokens_all_allowed": ok,
             "ms_per_step_reference_call_sequence": round(ms_ref, 3), "same_tokens_either_way": same,
+            "ms_per_step_library_gemms_only": round(ms_lib, 3), "tokens_equal_with_library_gemms": f"{equal_lib} of {S}",
             "ms_per_step_hip_graph_replay": ms_graph, "same_tokens_from_graph": same_graph,
             "config": {"workload": f"Llama-3-8B-shaped decode step, {layers} layers, 128 seqs, ctx U[1024,16384] "
                                    "(seed 5), bf16, per-layer paged KV"

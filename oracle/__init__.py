@@ -21,6 +21,8 @@ How each function is pinned (tests/test_oracle_*.py):
   rotary_embedding       closed form per element in fp64, norm preservation,
                          position 0 = identity, pass-through tail;
   rms_norm               closed form in fp64 incl. the round-then-scale order;
+  linear                 triple loop on small integers (exact), identity and
+                         one-hot weights, linearity in x;
   hostkv (allocator,     hand-computed cases from blocks.rs / batch_info.rs
   batch builder)         semantics plus exact agreement with the C++ core;
   aici bias              bit order from aicirt/src/api.rs:278-292 on hand cases;

@@ -314,6 +314,20 @@ def fused_add_rms_norm(input: torch.Tensor, residual: torch.Tensor, weight: torc
     input.copy_(normed * weight)
 
 
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+           residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`nn::Linear::forward` as built by llm/mod.rs:401-416 (`linear_no_bias`, `linear`): x . weight^T (+ bias),
+    weight [out, in] as a checkpoint stores it.  Computed in fp64 from the operands' own values and returned
+    in fp64 (a caller rounds, or bounds the distance).  With `residual`: the value rounded to x's dtype, plus
+    the residual, in fp64 -- the separate addition of llama.rs:166, 173 before its own rounding."""
+    y = x.double() @ weight.double().t()
+    if bias is not None:
+        y = y + bias.double()
+    if residual is not None:
+        y = y.to(x.dtype).double() + residual.double()
+    return y
+
+
 def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
     """activation_kernels.cu:9-26: T(silu(x1) in fp32) * x2 in T."""
     d = x.shape[-1] // 2

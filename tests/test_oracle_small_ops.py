@@ -219,3 +219,36 @@ def test_sample_reduces_to_known_procedures():
     draws = np.array([aici.sample(logits, bias, 0.8, 0.6, u) for u in (np.arange(n) + 0.5) / n])
     assert (kept[draws] > 0).all() and 0.6 <= kept.sum() < 0.6 + p.max()
     assert np.abs(np.bincount(draws, minlength=V) / n - kept / kept.sum()).max() < 1.5 / n + 1e-6
+
+
+def test_linear_against_a_triple_loop_and_closed_forms():
+    g = torch.Generator().manual_seed(11)
+    M, N, Kd = 5, 7, 6
+    # small integers: every product and sum is exact in any float type, so the comparison is exact
+    x = torch.randint(-4, 5, (M, Kd), generator=g).float()
+    w = torch.randint(-4, 5, (N, Kd), generator=g).float()
+    b = torch.randint(-4, 5, (N,), generator=g).float()
+    want = torch.zeros((M, N), dtype=torch.float64)
+    for i in range(M):
+        for j in range(N):
+            acc = 0.0
+            for k in range(Kd):
+                acc += float(x[i, k]) * float(w[j, k])  # weight is [out, in]: row j makes output j
+            want[i, j] = acc + float(b[j])
+    assert torch.equal(ref.linear(x, w, b), want)
+    assert torch.equal(ref.linear(x, w), want - b.double())
+    # identity weight returns x; a one-hot row picks a column of x; a transposed operand would fail both
+    xr = torch.randn((4, 6), generator=g)
+    assert torch.equal(ref.linear(xr, torch.eye(6)), xr.double())
+    pick = torch.zeros((2, 6))
+    pick[0, 4] = 1.0
+    pick[1, 1] = -2.0
+    assert torch.equal(ref.linear(xr, pick), torch.stack([xr[:, 4], -2.0 * xr[:, 1]], dim=1).double())
+    # linear in x
+    x2 = torch.randint(-4, 5, (M, Kd), generator=g).float()
+    assert torch.equal(ref.linear(x + x2, w), ref.linear(x, w) + ref.linear(x2, w))
+    # the residual is added to the value as the data type holds it
+    xb, wb = torch.randn((3, 8), generator=g).bfloat16(), torch.randn((4, 8), generator=g).bfloat16()
+    r = torch.randn((3, 4), generator=g).bfloat16()
+    y = ref.linear(xb, wb)
+    assert torch.equal(ref.linear(xb, wb, residual=r), y.to(torch.bfloat16).double() + r.double())
