@@ -3,14 +3,16 @@
 // `linear_no_bias`, llm/mod.rs:401-407; phi.rs:70-71, 99, 116-117 through `linear`, mod.rs:409-416), where every
 // element of W is used once per row of x and the time goes into reading W from HBM exactly once.
 //
-// Shape of the kernel: a workgroup of four wavefronts owns 64 (or 128) rows of W and a range of k; a wavefront
-// owns 16 (or 32) of those rows.  Per 32 values of k a wavefront loads its piece of W straight from global memory
-// into the A operand of v_mfma_f32_16x16x32 (lane l: row l % 16, the 8 values of k at 8 (l / 16): 64 contiguous
-// bytes per row and instruction, loaded with the non-temporal hint, eight such pieces in flight per wavefront)
-// and multiplies it with the eight 16-row tiles of x, which the workgroup keeps in LDS in operand order (a lane's
-// 16 bytes at its lane index: read without bank conflicts), three stages of 64 values of k, one barrier per stage.
-// The accumulators hold y transposed: lane l has rows 4 (l / 16) .. + 3 of its 16 columns of W -- four consecutive
-// outputs of one row of y.
+// Shape of the kernel: a workgroup of four (or eight) wavefronts owns 128 (64 .. 256) rows of W and a range of k; a
+// wavefront owns 32 (or 16) of those rows.  Per 32 values of k a wavefront loads its pieces of W straight from
+// global memory into the A operand of v_mfma_f32_16x16x32 (lane l: row l % 16, the 8 values of k at 8 (l / 16): 64
+// contiguous bytes per row and instruction, plain loads; the pieces of four to eight steps are in flight per wavefront, asked
+// for two steps at a time) and multiplies them with the eight 16-row tiles of x, which the workgroup keeps in LDS
+// in operand order (a lane's 16 bytes at its lane index: read without bank conflicts, one step ahead of the
+// MFMAs that use them), three stages of 64 values of k, one barrier per stage.  Rows of x reach LDS through
+// registers, asked for as far ahead as the pieces of W: a wavefront's loads complete in order, so anything closer
+// would drain the pieces of W at every stage.  The accumulators hold y transposed: lane l has rows 4 (l / 16) .. + 3
+// of its 16 rows of W -- four consecutive outputs of one row of y.
 //
 // When W has too few rows to occupy the device, the range of k is split between workgroups; each leaves its sums
 // in fp32 in operand order, and a second launch adds them up in a fixed order (no atomics: the same bits on every
@@ -61,6 +63,11 @@ struct LinMfma<bf16_t> {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
 };
+
+// A piece of W: a plain load.  The two 64-byte halves of a cache line are asked for by two instructions, and with
+// the read-once hint the line may be gone before the second one arrives (measured: 10 % slower on the shapes of a
+// decode step).
+__device__ __forceinline__ uint4 load_w(const void *p) { return *static_cast<const uint4 *>(p); }
 
 template <typename To, typename From>
 __device__ __forceinline__ To lin_cast(From v) {
@@ -159,7 +166,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void skinny_linear_kernel(const Line
 #pragma unroll
   for (int j = 0; j < kLinDepth; j++)
 #pragma unroll
-    for (int t = 0; t < NT; t++) wq[j][t] = load16_once(wrow[t] + (int64_t)j * kLinStepK);
+    for (int t = 0; t < NT; t++) wq[j][t] = load_w(wrow[t] + (int64_t)j * kLinStepK);
 #pragma unroll
   for (int i = 1; i <= kLinXAhead; i++) xq[i % kLinXAhead] = load_x(min(i, nchunks - 1));
   __builtin_amdgcn_sched_barrier(0);  // every load above is on its way before the first wait
@@ -208,7 +215,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void skinny_linear_kernel(const Line
         for (int jj = j - (kLinBunch - 1); jj <= j; jj++) {
           const int ahead = min(base + jj + kLinDepth, nsteps - 1);
 #pragma unroll
-          for (int t = 0; t < NT; t++) wq[jj][t] = load16_once(wrow[t] + (int64_t)ahead * kLinStepK);
+          for (int t = 0; t < NT; t++) wq[jj][t] = load_w(wrow[t] + (int64_t)ahead * kLinStepK);
         }
       }
       // Steps stay apart: nothing of a later step is moved in front of this one's MFMAs.
