@@ -748,24 +748,32 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void paged_decode_flat_kern
         const int blk = b_first + 2 * it;
         pair_compute<T, HD>(p, r, blk, blk + 1 < nblk, ctx, slope, qreg, m_run, l_run, acc);
       };
+      // The pairs of a full batch are visited in bit-reversed order (0, 16, 8, 24, 4, ...), not in the order of the
+      // table.  A sequence whose blocks lie in the pool in the order of their tokens -- what an allocator hands a
+      // fresh prompt -- would otherwise be streamed with one constant stride by every wavefront at once, which the
+      // memory system serves 5 % slower than scattered blocks (717 against 682 us on 128 x U[1k,16k] tokens; with
+      // this order 675 us for either).  Batches of fewer than 32 pairs keep the table's order.  The order is the
+      // same for every block size and launch, so results are too.
+      const bool full = nsub == 32;
+      auto pair_at = [&](int pos) -> int { return full ? (int)(__builtin_bitreverse32((unsigned)pos) >> 27) : pos; };
       if (HD <= 128) {
         PairRegs<HD> ra, rb;
-        issue(0, ra);
+        issue(pair_at(0), ra);
         // the loop on a 256-byte boundary: 1 % on the whole step against where it happened to fall
         asm volatile(".p2align 8");
-        for (int it = 0; it < nsub; it += 2) {
-          if (it + 1 < nsub) issue(it + 1, rb);
-          fold(it, ra);
-          if (it + 1 < nsub) {
-            if (it + 2 < nsub) issue(it + 2, ra);
-            fold(it + 1, rb);
+        for (int pos = 0; pos < nsub; pos += 2) {
+          if (pos + 1 < nsub) issue(pair_at(pos + 1), rb);
+          fold(pair_at(pos), ra);
+          if (pos + 1 < nsub) {
+            if (pos + 2 < nsub) issue(pair_at(pos + 2), ra);
+            fold(pair_at(pos + 1), rb);
           }
         }
       } else {  // two register sets of 256-element heads do not fit
-        for (int it = 0; it < nsub; it++) {
+        for (int pos = 0; pos < nsub; pos++) {
           PairRegs<HD> ra;
-          issue(it, ra);
-          fold(it, ra);
+          issue(pair_at(pos), ra);
+          fold(pair_at(pos), ra);
         }
       }
     }
