@@ -748,14 +748,17 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void paged_decode_flat_kern
         const int blk = b_first + 2 * it;
         pair_compute<T, HD>(p, r, blk, blk + 1 < nblk, ctx, slope, qreg, m_run, l_run, acc);
       };
-      // The pairs of a full batch are visited in bit-reversed order (0, 16, 8, 24, 4, ...), not in the order of the
-      // table.  A sequence whose blocks lie in the pool in the order of their tokens -- what an allocator hands a
-      // fresh prompt -- would otherwise be streamed with one constant stride by every wavefront at once, which the
-      // memory system serves 5 % slower than scattered blocks (717 against 682 us on 128 x U[1k,16k] tokens; with
-      // this order 675 us for either).  Batches of fewer than 32 pairs keep the table's order.  The order is the
-      // same for every block size and launch, so results are too.
-      const bool full = nsub == 32;
-      auto pair_at = [&](int pos) -> int { return full ? (int)(__builtin_bitreverse32((unsigned)pos) >> 27) : pos; };
+      // The pairs of a batch are visited in bit-reversed order (of 32: 0, 16, 8, 24, 4, ...), not in the order of
+      // the table; in a batch of fewer than 32 the largest power of two of them is, the rest follow in table order.
+      // A sequence whose blocks lie in the pool in the order of their tokens -- what an allocator hands a fresh
+      // prompt -- would otherwise be streamed with one constant stride by every wavefront at once, which the memory
+      // system serves 5 % slower than scattered blocks (717 against 682 us on 128 x U[1k,16k] tokens; with this
+      // order 670 us for either).  Which pair comes next is scalar arithmetic on the position in the batch -- the
+      // same at every block size and in every launch, so results are too.
+      const int pk = 31 - __builtin_clz((unsigned)nsub);  // the largest power of two within the batch
+      auto pair_at = [&](int pos) -> int {
+        return pos < (1 << pk) ? (int)((__builtin_bitreverse32((unsigned)pos) >> 1) >> (31 - pk)) : pos;
+      };
       if (HD <= 128) {
         PairRegs<HD> ra, rb;
         issue(pair_at(0), ra);
