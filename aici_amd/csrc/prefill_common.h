@@ -38,6 +38,7 @@ struct PrefillParams {
   int table_cols;
   int64_t num_blocks;
   int64_t kc_block, kc_head, vc_block, vc_head;  // cache strides in elements
+  int64_t total_k;  // rows of k / v (all sequences): bounds the byte offsets inside a sequence
   int block_log2;  // paged forms: log2 of the cache's block size (3, 4 or 5); every kernel but the four-wavefront one needs 4
   // out holds fp32 instead of the input type: the accumulators divided by the row sums, not rounded again
   // (for checking the kernel's arithmetic apart from the rounding of its output; o_row / o_head count floats).

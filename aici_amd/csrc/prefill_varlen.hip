@@ -784,27 +784,44 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   const uint32_t kd_off = (uint32_t)(((int64_t)kd_tok * p.k_row + kd_run * 8) * (int64_t)sizeof(T));
   const uint32_t kd_off_last =
       (uint32_t)(((int64_t)kd_tok * p.k_row + (min(4 * (KPB - 1) + kd_run, d_chunks - 1) - 4 * (KPB - 1)) * 8) * (int64_t)sizeof(T));
+  // The scalar side of a copy is kept short -- a wavefront issues its instructions in order, and every scalar
+  // instruction in front of a copy is time its vector block does not have: the base of the copies is the start
+  // of the sequence's keys (one scalar pointer for the whole loop), a tile's and a piece's place go into the
+  // lane's 32-bit byte offset (the host sends launches whose keys span more than that to the other kernel), and a
+  // piece's place in LDS is its number times 1 KiB.
+  constexpr int KW = (KNP + 7) / 8;  // pieces per wavefront
+  uint32_t k_off0[KW];
+  if constexpr (ROWS) {
+#pragma unroll
+    for (int i = 0; i < KW; i++) {
+      const int q = wave_u + 8 * i, r = q / KPB, pi = q % KPB;
+      k_off0[i] = (pi == KPB - 1 ? kd_off_last : kd_off) + (uint32_t)(((int64_t)16 * r * p.k_row + 32 * pi) * (int64_t)sizeof(T));
+    }
+  }
+  const T *kp_u = uniform_ptr(kp);
+  const T *vp_u = uniform_ptr(vp);
+  const uint32_t k_tile_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((int64_t)BN * p.k_row * (int64_t)sizeof(T)));
+  const uint32_t v_tile_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((int64_t)BN * p.v_row * (int64_t)sizeof(T)));
+  const unsigned lds_wave = (unsigned)__builtin_amdgcn_readfirstlane(
+      (int)((unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem_raw + (unsigned)wave_u * 1024u));
   auto k_rows_dma = [&](int tile) {
     const int k0 = tile * BN;
-    const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem_raw;
+    const unsigned dst0 = lds_wave + (unsigned)((tile % NST) * STAGE_ELEMS * (int)sizeof(T));
+    const uint32_t tile_off = (uint32_t)tile * k_tile_bytes;
 #pragma unroll
-    for (int i = 0; i < (KNP + 7) / 8; i++) {
+    for (int i = 0; i < KW; i++) {
       const int q = wave_u + 8 * i;
       if (KNP % 8 == 0 || q < KNP) {
-        const int r = q / KPB, pi = q % KPB;
-        uint32_t off = pi == KPB - 1 ? kd_off_last : kd_off;
-        int64_t first = (int64_t)(k0 + 16 * r) * p.k_row + 32 * pi;  // elements from kp; uniform
+        uint32_t off = k_off0[i] + tile_off;
         if (k0 + BN > Lk) {
+          const int r = q / KPB, pi = q % KPB;
           const int key = min(k0 + 16 * r + kd_tok, Lk - 1);
-          off = (uint32_t)(((int64_t)(key - k0) * p.k_row + (min(4 * pi + kd_run, d_chunks - 1) - 4 * pi) * 8) * (int64_t)sizeof(T));
-          first = (int64_t)k0 * p.k_row + 32 * pi;
+          off = (uint32_t)(((int64_t)key * p.k_row + min(4 * pi + kd_run, d_chunks - 1) * 8) * (int64_t)sizeof(T));
         }
-        const T *src = uniform_ptr(kp + first);
-        const unsigned dst = (unsigned)__builtin_amdgcn_readfirstlane(
-            (int)(lds_base + (unsigned)(((tile % NST) * STAGE_ELEMS + r * (HDP * 16)) * (int)sizeof(T)) + pi * 1024));
+        const unsigned dst = dst0 + (unsigned)i * 8192u;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                      :
-                     : "s"(dst), "v"(off), "s"(src)
+                     : "s"(dst), "v"(off), "s"(kp_u)
                      : "memory", "m0");
       }
     }
@@ -831,13 +848,13 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
   }
   auto v_rows_dma = [&](int tile) {
     const int k0 = tile * BN;
-    const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem_raw;
-    const T *src = uniform_ptr(vp + (int64_t)k0 * p.v_row);
+    const unsigned dst0 = lds_wave + (unsigned)(((tile % NST) * STAGE_ELEMS + K_ELEMS) * (int)sizeof(T));
+    const uint32_t tile_off = (uint32_t)tile * v_tile_bytes;
 #pragma unroll
     for (int i = 0; i < VNPW; i++) {
       const int q = wave_u + 8 * i;
       if (VNP % 8 == 0 || q < VNP) {
-        uint32_t off = vd_off[i];
+        uint32_t off = vd_off[i] + tile_off;
         if (k0 + BN > Lk) {
           // (the lane number through an opaque copy: hoisted out of the loop, what is derived from it here
           // would hold registers that the loop does not have)
@@ -845,13 +862,12 @@ __global__ __launch_bounds__(512, 2) void prefill_varlen_w8_kernel(PrefillParams
           asm volatile("" : "+v"(l2));
           const int u = q * 64 + l2;
           const int r = u / CPRV, pc = u % CPRV;
-          off = (uint32_t)(((int64_t)(min(k0 + r, Lk - 1) - k0) * p.v_row + min(pc ^ vswz(r), d_chunks - 1) * 8) * (int64_t)sizeof(T));
+          off = (uint32_t)(((int64_t)min(k0 + r, Lk - 1) * p.v_row + min(pc ^ vswz(r), d_chunks - 1) * 8) * (int64_t)sizeof(T));
         }
-        const unsigned dst = (unsigned)__builtin_amdgcn_readfirstlane(
-            (int)(lds_base + (unsigned)(((tile % NST) * STAGE_ELEMS + K_ELEMS) * (int)sizeof(T)) + q * 1024));
+        const unsigned dst = dst0 + (unsigned)i * 8192u;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                      :
-                     : "s"(dst), "v"(off), "s"(src)
+                     : "s"(dst), "v"(off), "s"(vp_u)
                      : "memory", "m0");
       }
     }
@@ -1373,7 +1389,10 @@ void pick_qt(const PrefillParams &p, int64_t total_q, hipStream_t stream) {
   if constexpr (HDP <= 128) {
     const int force = tuning().prefill_kernel;  // 0: choose here; 1: eight wavefronts; 2 / 3: four wavefronts, 2 / 1 row tiles
     // the eight-wavefront kernel addresses a tile's 64 rows with unsigned 32-bit byte offsets
-    const bool fits = p.k_row >= 0 && p.k_row < (1 << 23) && p.v_row >= 0 && p.v_row < (1 << 23);
+    // ... and a sequence's keys and values with unsigned 32-bit byte offsets from its first row
+    const int64_t span = (int64_t)1 << 32;
+    const bool fits = p.k_row >= 0 && p.v_row >= 0 && (p.total_k + 64) * p.k_row * (int64_t)sizeof(T) < span &&
+                      (p.total_k + 64) * p.v_row * (int64_t)sizeof(T) < span;
     // it knows the causal mask and no mask; other windows go to the four-wavefront kernel
     const bool plain = p.win_left < 0 && p.win_right <= 0;
     if (plain && fits && (force == 0 || force == 1)) {
@@ -1509,6 +1528,7 @@ void mha_varlen_fwd_impl(const hipattn_tensor *q, const hipattn_tensor *k, const
   p.cu_q = static_cast<const int32_t *>(cu_q->data);
   p.cu_k = static_cast<const int32_t *>(cu_k->data);
   p.seqused_k = seqused_k ? static_cast<const int32_t *>(seqused_k->data) : nullptr;
+  p.total_k = k->sizes[0];
   p.batch = batch;
   p.Hq = Hq;
   p.Hkv = Hkv;

@@ -140,6 +140,33 @@ def test_strided_qkv_from_a_fused_projection(device):
     assert (got.cpu().double() - fp64(p)).abs().max().item() <= TOL[dtype]
 
 
+def test_rows_too_far_apart_for_32_bit_offsets(device):
+    """The eight-wavefront kernel addresses a sequence's keys with 32-bit byte offsets from its first row; k / v
+    whose rows span 4 GiB or more (here: views of a buffer with 8 MiB between rows) go to the other kernel."""
+    lens = [200, 300]
+    p = general_inputs(31, lens, lens, 4, 2, 64, torch.bfloat16)
+    want = fp64(p)
+    T, pitch = sum(lens), 1 << 22
+    qd, cu = p.q.to(device), p.cu_q.to(device)
+    wide_k = torch.zeros((T, pitch), dtype=torch.bfloat16, device=device)  # 4 GiB
+    wide_k[:, :128] = p.k.reshape(T, 128).to(device)
+    kd = wide_k[:, :128].view(T, 2, 64)
+    assert kd.stride(0) == pitch and (T + 64) * pitch * 2 >= 1 << 32
+    out = K.flash_attn_varlen(qd, kd, p.v.to(device), cu, cu, p.max_q, p.max_k, p.scale, True)
+    assert (out.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16]
+    del wide_k, kd
+    wide_v = torch.zeros((T, pitch), dtype=torch.bfloat16, device=device)
+    wide_v[:, :128] = p.v.reshape(T, 128).to(device)
+    vd = wide_v[:, :128].view(T, 2, 64)
+    out = K.flash_attn_varlen(qd, p.k.to(device), vd, cu, cu, p.max_q, p.max_k, p.scale, True)
+    assert (out.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16]
+    # just inside the limit: the same rows 2 MiB apart stay with the eight-wavefront kernel
+    near = torch.zeros((T, 1 << 20), dtype=torch.bfloat16, device=device)
+    near[:, :128] = p.k.reshape(T, 128).to(device)
+    out = K.flash_attn_varlen(qd, near[:, :128].view(T, 2, 64), p.v.to(device), cu, cu, p.max_q, p.max_k, p.scale, True)
+    assert (out.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16]
+
+
 def test_random_ragged_cases(device):
     """Twenty-four seeded draws of dtype, head shape (sizes that fill their MFMA tiles and sizes that do not),
     batch, new and prior lengths around the tile sizes (1, 63..65, 255..257, 513) and mask, against the fp32
