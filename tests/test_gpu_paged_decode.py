@@ -175,6 +175,32 @@ def test_invariant_under_block_permutation_and_equals_prefill_last_row(device):
     assert (pre[-1].cpu().float() - got[s].float()).abs().max().item() <= 2e-2
 
 
+def test_blocks_in_token_order_and_scattered_give_the_same_bits_on_long_contexts(device, tuning):
+    """A wavefront visits the block pairs of a batch in an order of its own (bit-reversed positions), which depends
+    on the position in the context alone: the same keys give the same bits wherever their blocks lie -- in the pool
+    in token order, as an allocator hands them to a fresh prompt, or scattered -- and the values are the oracle's.
+    Contexts long enough for full batches of 32 pairs and for ragged ends, flat split and partitioned launch."""
+    dtype = torch.bfloat16
+    c = W.decode_inputs(23, 12, 1500, 5000, 32, 8, 128, dtype, 3000)
+    nb = (c.context_lens.numpy().astype(np.int64) + 15) // 16
+    order = np.zeros(tuple(c.block_tables.shape), dtype=np.int64)
+    start = 0
+    for s_, n in enumerate(nb):
+        order[s_, :n] = np.arange(start, start + n)
+        start += int(n)
+    kc2, vc2 = torch.zeros_like(c.key_cache), torch.zeros_like(c.value_cache)
+    for s_, n in enumerate(nb):  # the same keys and values, moved to blocks 0, 1, 2, ... in token order
+        kc2[order[s_, :n]] = c.key_cache[c.block_tables[s_, :n].long()]
+        vc2[order[s_, :n]] = c.value_cache[c.block_tables[s_, :n].long()]
+    c2 = W.DecodeInputs(c.q, kc2, vc2, torch.from_numpy(order.astype(np.int32)), c.context_lens, c.max_ctx, c.scale, 8)
+    want = ref.paged_attention_fp64(c.q, c.key_cache, c.value_cache, 8, c.scale, c.block_tables, c.context_lens, 16)
+    for flat in (1, 0):
+        tuning("decode_flat", flat)
+        a, b = run_v1(c, device), run_v1(c2, device)
+        assert torch.equal(a, b)
+        assert (a.cpu().double() - want).abs().max().item() <= TOL[dtype]
+
+
 def test_config2_full_size(device):
     """The benchmark's decode configuration at full size: every one of the 64 sequences against the float64
     statement of the oracle, and every third one against the slot-by-slot oracle itself."""
