@@ -94,6 +94,8 @@ _ERR_FUNCS = {
     "hipattn_fused_add_rms_norm": [TP, TP, TP, c_float, c_void_p],
     "hipattn_linear": [TP, TP, TP, TP, TP, TP, c_void_p],
     "hipattn_linear_workspace_size": [TP, TP, POINTER(c_int64)],
+    "hipattn_linear_rms_norm": [TP, TP, TP, TP, TP, TP, TP, c_float, TP, c_void_p],
+    "hipattn_linear_rms_norm_workspace_size": [TP, TP, POINTER(c_int64)],
     "hipattn_silu_and_mul": [TP, TP, c_void_p],
     "hipattn_gelu_new": [TP, TP, c_void_p],
     "hipattn_gelu_fast": [TP, TP, c_void_p],

@@ -96,4 +96,27 @@ __device__ __forceinline__ V bit_cast(const U &u) {
   return v;
 }
 
+// Sums over a wavefront and over the workgroup (every thread receives the result); the order of the additions
+// is fixed by the thread numbers alone, so two kernels that hand these the same per-thread values get the same
+// bits.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float block_sum(float v, float *smem /* >= 17 floats */) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nwaves = (blockDim.x + 63) >> 6;
+  v = wave_sum(v);
+  if (lane == 0) smem[wave] = v;
+  __syncthreads();
+  if (wave == 0) {
+    float t = lane < nwaves ? smem[lane] : 0.f;
+    t = wave_sum(t);
+    if (lane == 0) smem[16] = t;
+  }
+  __syncthreads();
+  return smem[16];
+}
+
 }  // namespace hipattn

@@ -9,28 +9,6 @@ namespace hipattn {
 
 namespace {
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
-
-// Sum over the workgroup; every thread receives the result.
-__device__ __forceinline__ float block_sum(float v, float *smem /* >= 17 floats */) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int nwaves = (blockDim.x + 63) >> 6;
-  v = wave_sum(v);
-  if (lane == 0) smem[wave] = v;
-  __syncthreads();
-  if (wave == 0) {
-    float t = lane < nwaves ? smem[lane] : 0.f;
-    t = wave_sum(t);
-    if (lane == 0) smem[16] = t;
-  }
-  __syncthreads();
-  return smem[16];
-}
-
 // ---------------------------------------------------------------------------
 // rotary_embedding (pos_encoding_kernels.cu:9-77).  Every product and the
 // final sum are rounded to T, which is what the reference's per-operator

@@ -47,6 +47,13 @@ struct LinearParams {
   int mtiles;  // ceil(M / 16)
   int64_t ldx, ldw, ldr, ldo;
   int splits, steps_per_split, total_steps;
+  // with an RMS norm behind the layer: the sums go to the workspace as rows ([range][128 rows][N] fp32), and the
+  // launch that adds them up also normalises the finished row
+  int row_sums;
+  const void *norm_w;
+  void *norm_out;
+  int64_t ldn;
+  float eps;
 };
 
 template <typename T>
@@ -223,7 +230,19 @@ __global__ __launch_bounds__(WAVES * 64, 2) void skinny_linear_kernel(const Line
     }
   }
 
-  if (p.splits == 1) {
+  if (p.row_sums) {
+    // rows of fp32 sums, one 16-byte piece per lane and tile (four lanes make 64 contiguous bytes of a row)
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+      const int n = n_wave + t * 16 + 4 * kg;
+      if (n < p.N) {
+#pragma unroll
+        for (int mt = 0; mt < kLinMT; mt++)
+          if (mt < p.mtiles)
+            *reinterpret_cast<f32x4_t *>(p.partial + ((int64_t)split * kLinMaxRows + mt * 16 + col) * p.N + n) = acc[t][mt];
+      }
+    }
+  } else if (p.splits == 1) {
 #pragma unroll
     for (int t = 0; t < NT; t++)
 #pragma unroll
@@ -262,6 +281,69 @@ __global__ __launch_bounds__(256) void skinny_linear_reduce_kernel(const LinearP
     for (int r = 0; r < 4; r++) s[r] += v[r];
   }
   linear_finish<T>(p, s, mt * 16 + (lane & 15), (int)nt * 16 + 4 * (lane >> 4));
+}
+
+// Adds up the ranges' sums of one row of y, finishes the row (bias, rounding, residual: as linear_finish) and
+// applies the RMS norm that follows the layer (llama.rs:165, 169, 207 behind 166, 173) in the same launch: one
+// workgroup per row, a thread's eight columns stay in registers between the two.  The norm's arithmetic and the
+// order of its additions are those of the stand-alone kernel (rms_norm_vec8_kernel: the same thread owns the same
+// eight columns, the same block_sum), so the two routes give the same bits.
+template <typename T>
+__global__ __launch_bounds__(1024) void skinny_linear_reduce_norm_kernel(const LinearParams p) {
+  __shared__ float smem[17];
+  const int row = blockIdx.x;
+  const int i = threadIdx.x * 8;
+  const bool active = i < p.N;
+  float v[8];
+  float ss = 0.f;
+  if (active) {
+    const float *src = p.partial + (int64_t)row * p.N + i;
+    const int64_t stride = (int64_t)kLinMaxRows * p.N;
+    f32x4_t a = *reinterpret_cast<const f32x4_t *>(src), b = *reinterpret_cast<const f32x4_t *>(src + 4);
+    for (int k = 1; k < p.splits; k++) {
+      const f32x4_t a2 = *reinterpret_cast<const f32x4_t *>(src + k * stride);
+      const f32x4_t b2 = *reinterpret_cast<const f32x4_t *>(src + k * stride + 4);
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        a[r] += a2[r];
+        b[r] += b2[r];
+      }
+    }
+    const T *bias = static_cast<const T *>(p.bias);
+    const T *res = static_cast<const T *>(p.residual);
+    uint4 braw = make_uint4(0, 0, 0, 0), rraw = braw, oraw;
+    if (bias != nullptr) braw = *reinterpret_cast<const uint4 *>(bias + i);
+    if (res != nullptr) rraw = *reinterpret_cast<const uint4 *>(res + (int64_t)row * p.ldr + i);
+    const T *be = reinterpret_cast<const T *>(&braw);
+    const T *re = reinterpret_cast<const T *>(&rraw);
+    T *oe = reinterpret_cast<T *>(&oraw);
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      float f = j < 4 ? a[j] : b[j - 4];
+      if (bias != nullptr) f += to_float(be[j]);
+      T y = from_float<T>(f);
+      if (res != nullptr) y = add_t<T>(y, re[j]);
+      oe[j] = y;
+      v[j] = to_float(y);
+    }
+    *reinterpret_cast<uint4 *>(static_cast<T *>(p.out) + (int64_t)row * p.ldo + i) = oraw;
+#pragma unroll
+    for (int j = 0; j < 8; j++) ss += v[j] * v[j];
+  }
+  const float total = block_sum(ss, smem);
+  const float inv = rsqrtf(total / (float)p.N + p.eps);
+  if (active) {
+    const uint4 wr = *reinterpret_cast<const uint4 *>(static_cast<const T *>(p.norm_w) + i);
+    const T *we = reinterpret_cast<const T *>(&wr);
+    uint4 o;
+    T *oe = reinterpret_cast<T *>(&o);
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const T normed = from_float<T>(v[j] * inv);
+      oe[j] = from_float<T>(to_float(normed) * to_float(we[j]));
+    }
+    *reinterpret_cast<uint4 *>(static_cast<T *>(p.norm_out) + (int64_t)row * p.ldn + i) = o;
+  }
 }
 
 struct LinearPlan {
@@ -308,7 +390,12 @@ void launch_linear(const LinearParams &p, const LinearPlan &pl, hipStream_t stre
   else
     hipLaunchKernelGGL((skinny_linear_kernel<T, 1, 8, 4>), grid, block, 0, stream, p);
   check_launch("linear");
-  if (pl.splits > 1) {
+  if (p.row_sums) {
+    int threads = (int)(((p.N / 8 + 63) / 64) * 64);
+    if (threads > 1024) threads = 1024;  // (the entry point bounds N)
+    hipLaunchKernelGGL((skinny_linear_reduce_norm_kernel<T>), dim3((unsigned)p.M), dim3((unsigned)threads), 0, stream, p);
+    check_launch("linear (sum of the ranges + rms_norm)");
+  } else if (pl.splits > 1) {
     const int64_t threads = (int64_t)((p.N + 15) / 16) * p.mtiles * 64;
     hipLaunchKernelGGL((skinny_linear_reduce_kernel<T>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, p);
     check_launch("linear (sum of the splits)");
@@ -317,8 +404,12 @@ void launch_linear(const LinearParams &p, const LinearPlan &pl, hipStream_t stre
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// With `norm_out` the RMS norm of the finished rows (weight `norm_weight`, `eps`) is written there by the launch
+// that adds up the ranges' sums; the workspace is then needed whatever the number of ranges.
 void linear_impl(hipattn_tensor *out, const hipattn_tensor *x, const hipattn_tensor *weight, const hipattn_tensor *bias,
-                 const hipattn_tensor *residual, const hipattn_tensor *workspace, void *stream_arg, int64_t *ws_query) {
+                 const hipattn_tensor *residual, const hipattn_tensor *workspace, void *stream_arg, int64_t *ws_query,
+                 hipattn_tensor *norm_out = nullptr, const hipattn_tensor *norm_weight = nullptr, float eps = 0.f,
+                 bool ws_query_with_norm = false) {
   check_tensor(x, "x", 2);
   check_tensor(weight, "weight", 2);
   const int dt = x->dtype;
@@ -332,7 +423,10 @@ void linear_impl(hipattn_tensor *out, const hipattn_tensor *x, const hipattn_ten
            kLinGroupK);
   HA_CHECK(N % 16 == 0, "linear: the number of rows of weight (%lld) must be a multiple of 16", (long long)N);
   HA_CHECK(N < (1 << 24) && K < (1 << 24), "linear: sizes out of range");
-  const LinearPlan pl = plan_linear((int)M, (int)N, (int)K);
+  LinearPlan pl = plan_linear((int)M, (int)N, (int)K);
+  const bool with_norm = norm_out != nullptr || ws_query_with_norm;
+  // rows of sums for the norm: [range][128 rows][N] fp32 -- the size the tiles of sums take as well
+  if (with_norm) pl.partial_bytes = (size_t)pl.splits * kLinMaxRows * (size_t)N * sizeof(float);
   if (ws_query != nullptr) {
     *ws_query = (int64_t)pl.partial_bytes;
     return;
@@ -381,11 +475,34 @@ void linear_impl(hipattn_tensor *out, const hipattn_tensor *x, const hipattn_ten
     p.residual = residual->data;
     p.ldr = residual->strides[0];
   }
+  if (with_norm) {
+    HA_CHECK(N % 8 == 0 && N <= 8192, "linear_rms_norm: the number of rows of weight (%lld) must be a multiple of 8, at most 8192",
+             (long long)N);
+    check_tensor(norm_out, "norm_out", 2);
+    HA_CHECK(norm_weight != nullptr, "linear_rms_norm: norm_weight is NULL");
+    check_tensor(norm_weight, "norm_weight", 1);
+    HA_CHECK(norm_out->dtype == dt && norm_out->sizes[0] == M && norm_out->sizes[1] == N && norm_out->strides[1] == 1,
+             "linear_rms_norm: norm_out must be [%lld, %lld] %s with a contiguous last dimension", (long long)M, (long long)N,
+             dtype_name(dt));
+    HA_CHECK(norm_weight->dtype == dt && norm_weight->sizes[0] == N && norm_weight->strides[0] == 1,
+             "linear_rms_norm: norm_weight must be %lld contiguous %s", (long long)N, dtype_name(dt));
+    check_data(norm_out, "norm_out");
+    check_data(norm_weight, "norm_weight");
+    HA_CHECK(out->strides[0] % 8 == 0 && norm_out->strides[0] % 8 == 0 && aligned16(out->data) && aligned16(norm_out->data) &&
+                 aligned16(norm_weight->data) && (bias == nullptr || aligned16(bias->data)) &&
+                 (residual == nullptr || (residual->strides[0] % 8 == 0 && aligned16(residual->data))),
+             "linear_rms_norm: rows of out, norm_out and residual, and bias and norm_weight, must start on 16-byte boundaries");
+    p.row_sums = 1;
+    p.norm_w = norm_weight->data;
+    p.norm_out = norm_out->data;
+    p.ldn = norm_out->strides[0];
+    p.eps = eps;
+  }
   p.splits = pl.splits;
   p.steps_per_split = pl.steps_per_split;
   p.total_steps = (int)(K / kLinStepK);
   hipStream_t stream = resolve_stream(stream_arg);
-  if (pl.splits > 1) {
+  if (pl.splits > 1 || with_norm) {
     if (workspace != nullptr) {
       check_tensor(workspace, "workspace", 1);
       HA_CHECK(workspace->dtype == HIPATTN_U8 && workspace->strides[0] == 1, "linear: workspace must be contiguous u8");
@@ -419,5 +536,23 @@ extern "C" char *hipattn_linear_workspace_size(const hipattn_tensor *x, const hi
   HA_PROTECT({
     HA_CHECK(bytes != nullptr, "linear_workspace_size: bytes is NULL");
     linear_impl(nullptr, x, weight, nullptr, nullptr, nullptr, nullptr, bytes);
+  });
+}
+
+extern "C" char *hipattn_linear_rms_norm(hipattn_tensor *out, hipattn_tensor *norm_out, const hipattn_tensor *x,
+                                         const hipattn_tensor *weight, const hipattn_tensor *bias,
+                                         const hipattn_tensor *residual, const hipattn_tensor *norm_weight, float epsilon,
+                                         const hipattn_tensor *workspace, void *stream) {
+  HA_PROTECT({
+    HA_CHECK(norm_out != nullptr, "linear_rms_norm: norm_out is NULL");
+    linear_impl(out, x, weight, bias, residual, workspace, stream, nullptr, norm_out, norm_weight, epsilon);
+  });
+}
+
+extern "C" char *hipattn_linear_rms_norm_workspace_size(const hipattn_tensor *x, const hipattn_tensor *weight,
+                                                        int64_t *bytes) {
+  HA_PROTECT({
+    HA_CHECK(bytes != nullptr, "linear_rms_norm_workspace_size: bytes is NULL");
+    linear_impl(nullptr, x, weight, nullptr, nullptr, nullptr, nullptr, bytes, nullptr, nullptr, 0.f, true);
   });
 }

@@ -268,6 +268,25 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     return out
 
 
+def linear_rms_norm(x: torch.Tensor, weight: torch.Tensor, norm_weight: torch.Tensor, epsilon: float,
+                    bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None,
+                    workspace: Optional[torch.Tensor] = None):
+    """`linear` and the RMS norm of its rows in the launch that finishes them: returns (out, rms_norm(out)),
+    the same bits as `linear` followed by `rms_norm`."""
+    out = torch.empty((x.size(0), weight.size(0)), dtype=x.dtype, device=x.device)
+    normed = torch.empty_like(out)
+    call("hipattn_linear_rms_norm", _desc(out, "out"), _desc(normed, "norm_out"), _desc(x, "x"), _desc(weight, "weight"),
+         _desc(bias, "bias"), _desc(residual, "residual"), _desc(norm_weight, "norm_weight"), float(epsilon),
+         _desc(workspace, "workspace"), _stream(x))
+    return out, normed
+
+
+def linear_rms_norm_workspace_size(x: torch.Tensor, weight: torch.Tensor) -> int:
+    n = ctypes.c_int64(0)
+    call("hipattn_linear_rms_norm_workspace_size", _desc(x, "x"), _desc(weight, "weight"), ctypes.byref(n))
+    return int(n.value)
+
+
 def linear_workspace_size(x: torch.Tensor, weight: torch.Tensor) -> int:
     n = ctypes.c_int64(0)
     call("hipattn_linear_workspace_size", _desc(x, "x"), _desc(weight, "weight"), ctypes.byref(n))

@@ -6,7 +6,8 @@ model :201-213) followed by the AICI logit-mask + greedy step
 The embedding is a library gather and the projections are library GEMMs (torch on
 ROCm) -- except, in a step of at most 128 rows, the two projections that close a
 residual branch (o_proj, down_proj): those go through the C ABI's linear kernel, which
-splits the inner dimension over the device and adds the residual in its epilogue.
+splits the inner dimension over the device and finishes the rows -- residual and the RMS
+norm that follows -- in the launch that adds the parts up.
 Everything else -- rms_norm, rotary, the paged-KV attention composition,
 silu_and_mul, bias + argmax -- goes through the C ABI as well.  Weights are random
 (there are no checkpoints here): the harness measures and checks the step's
@@ -89,6 +90,7 @@ class Llama:
         self.cfg = cfg
         self.device = device
         self.skinny_linear = True  # False: every projection is a library GEMM
+        self.fused_norm = True     # False: the norm behind those projections is a launch of its own
         w = {k: v.to(device) for k, v in weights.items()}
         self.wte = w["model.embed_tokens"]
         self.ln_f = w["model.norm"]
@@ -113,13 +115,19 @@ class Llama:
         kernels.rms_norm(out, x, weight, self.cfg.rms_norm_eps)
         return out
 
-    def _proj_add(self, y: torch.Tensor, weight: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
-        """y @ weight.T + x (llama.rs:96 + 166, 143 + 173).  Few rows and a weight with few of them (the shapes
-        on which a library GEMM leaves most of the device idle): the C ABI's kernel; else a library GEMM and
-        an addition."""
+    def _proj_add_norm(self, y: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tensor):
+        """x' = y @ weight.T + x (llama.rs:96 + 166, 143 + 173) and the RMS norm of x' that follows it (:169, :165 of the
+        next block, :207).  Few rows and a weight with few of them (the shapes on which a library GEMM leaves most
+        of the device idle): the C ABI's kernel, which splits the inner dimension over the device and finishes the
+        rows -- residual and norm -- in the launch that adds the parts up; else a library GEMM, an addition and
+        rms_norm.  The same bits either way as far as the norm goes."""
         if self.skinny_linear and weight.size(0) <= 8192 and kernels.linear_takes(y, weight):
-            return kernels.linear(y, weight, residual=x)
-        return y @ weight.t() + x
+            if self.fused_norm:
+                return kernels.linear_rms_norm(y, weight, norm_weight, self.cfg.rms_norm_eps, residual=x)
+            x = kernels.linear(y, weight, residual=x)
+            return x, self._rms(x, norm_weight)
+        x = y @ weight.t() + x
+        return x, self._rms(x, norm_weight)
 
     def forward(self, batch_info: BatchInfo, caches: List[Tuple[torch.Tensor, torch.Tensor]],
                 paged_prefill: bool = False, fused: bool = False) -> torch.Tensor:
@@ -131,8 +139,8 @@ class Llama:
         Hq, Hkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
         x = self.wte.index_select(0, batch_info.tokens.long())                   # llama.rs:203
         T = x.size(0)
-        for layer, (kc, vc) in zip(self.layers, caches):
-            h = self._rms(x, layer["rms_1"])                                    # :165
+        h = self._rms(x, self.layers[0]["rms_1"])                               # :165
+        for li, (layer, (kc, vc)) in enumerate(zip(self.layers, caches)):
             qkv = h @ layer["qkv"].t()                                          # :81-83
             if fused:
                 q, k, v = qkv.split([Hq * d, Hkv * d, Hkv * d], dim=1)
@@ -144,13 +152,14 @@ class Llama:
                 q, k, v = (t.contiguous() for t in qkv.split([Hq * d, Hkv * d, Hkv * d], dim=1))
                 q, k = self.rotary.forward(batch_info.positions, q, k)          # :85 (in place on the copies)
                 y = varlen_attn(q, k, v.reshape(T, Hkv, d), batch_info, kc, vc, paged_prefill=paged_prefill)  # :93
-            x = self._proj_add(y, layer["o"], x)                                 # :96, :166
-            h = self._rms(x, layer["rms_2"])                                    # :169
+            x, h = self._proj_add_norm(y, layer["o"], x, layer["rms_2"])         # :96, :166, :169
             gu = h @ layer["gate_up"].t()                                       # :135-136
             act = torch.empty((T, cfg.intermediate_size), dtype=x.dtype, device=x.device)
             kernels.silu_and_mul(act, gu)                                       # :140-142
-            x = self._proj_add(act, layer["down"], x)                            # :143, :173
-        x0 = self._rms(x, self.ln_f)                                            # :207
+            # the norm behind the block is the next block's first one, or the model's last (:165, :207)
+            after = self.layers[li + 1]["rms_1"] if li + 1 < len(self.layers) else self.ln_f
+            x, h = self._proj_add_norm(act, layer["down"], x, after)            # :143, :173
+        x0 = h
         sel = x0.index_select(0, batch_info.logit_idxs.long())                  # :209 extract_positions
         return sel @ self.lm_head.t()                                           # :210
 

@@ -319,6 +319,28 @@ char *hipattn_linear_workspace_size(const hipattn_tensor *x,
                                     const hipattn_tensor *weight,
                                     int64_t *bytes);
 
+/* hipattn_linear followed by the RMS norm of the finished rows, in the launch
+ * that adds up the ranges of the inner dimension: out = x . weight^T (+ bias)
+ * (+ residual) as above, norm_out = rms_norm(out, norm_weight, epsilon) with the
+ * arithmetic of hipattn_rms_norm -- the same bits as the two calls one after
+ * the other.  It is the pair that closes every residual branch of the decoder
+ * (llama.rs:166 + 169, 173 + 165 of the next block, 173 + 207), with no
+ * counterpart of its own in the reference's extern "C" block.  Operands as
+ * for hipattn_linear, and: N a multiple of 8, at most 8192; norm_weight [N],
+ * norm_out [M, N]; rows of out, norm_out and residual on 16-byte boundaries.
+ * The workspace (hipattn_linear_rms_norm_workspace_size bytes, or the
+ * library's per-stream scratch when NULL) is used whatever the shape. */
+char *hipattn_linear_rms_norm(hipattn_tensor *out, hipattn_tensor *norm_out,
+                              const hipattn_tensor *x,
+                              const hipattn_tensor *weight,
+                              const hipattn_tensor *bias,
+                              const hipattn_tensor *residual,
+                              const hipattn_tensor *norm_weight, float epsilon,
+                              const hipattn_tensor *workspace, void *stream);
+char *hipattn_linear_rms_norm_workspace_size(const hipattn_tensor *x,
+                                             const hipattn_tensor *weight,
+                                             int64_t *bytes);
+
 /* Replace silu_and_mul_C / gelu_new_C / gelu_fast_C (lib.rs:162-166;
  * activation_kernels.cu:15-115). */
 char *hipattn_silu_and_mul(hipattn_tensor *out, const hipattn_tensor *input,

@@ -145,6 +145,42 @@ def test_workspace_from_the_caller(device):
     assert K.linear_workspace_size(xd, wd) == 0
 
 
+@pytest.mark.parametrize("splits", [0, 1, 3, 8])
+def test_linear_rms_norm_gives_the_bits_of_the_two_calls(device, splits):
+    K.tuning_set("linear_splits", splits)
+    for (M, N, Kd, dtype, with_bias) in [(128, 4096, 4096, torch.bfloat16, False), (128, 4096, 14336, torch.bfloat16, False),
+                                         (37, 2560, 2560, torch.float16, True), (5, 64, 256, torch.bfloat16, True),
+                                         (128, 8192, 512, torch.bfloat16, False)]:
+        x, w, g = operands(M, N, Kd, dtype, seed=N + Kd + splits)
+        res = torch.randn((M, N), generator=g).to(dtype).to(device)
+        bias = torch.randn((N,), generator=g).to(dtype).to(device) if with_bias else None
+        nw = (1.0 + 0.1 * torch.randn((N,), generator=g)).to(dtype).to(device)
+        xd, wd = x.to(device), w.to(device)
+        out, normed = K.linear_rms_norm(xd, wd, nw, 1e-5, bias=bias, residual=res)
+        want = K.linear(xd, wd, bias=bias, residual=res)
+        assert torch.equal(out, want)
+        want_n = torch.empty_like(want)
+        K.rms_norm(want_n, want, nw, 1e-5)
+        assert torch.equal(normed, want_n)
+        # and the norm is the oracle's, from the rounded rows
+        o = ref.rms_norm(out.cpu(), nw.cpu(), 1e-5)
+        assert (normed.cpu().float() - o.float()).abs().max().item() <= (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10) * max(1.0, o.float().abs().max().item())
+    # without a residual, from the caller's workspace, and what is refused
+    x, w, g = operands(64, 1024, 768, torch.bfloat16, seed=77)
+    nw = torch.ones((1024,), dtype=torch.bfloat16, device=device)
+    xd, wd = x.to(device), w.to(device)
+    ws = torch.empty((K.linear_rms_norm_workspace_size(xd, wd),), dtype=torch.uint8, device=device)
+    assert ws.numel() > 0
+    out, normed = K.linear_rms_norm(xd, wd, nw, 1e-6, workspace=ws)
+    assert torch.equal(out, K.linear(xd, wd))
+    with pytest.raises(HipAttnError, match="at most 8192"):
+        K.linear_rms_norm(torch.zeros((8, 256), dtype=torch.bfloat16, device=device),
+                          torch.zeros((8208, 256), dtype=torch.bfloat16, device=device),
+                          torch.ones((8208,), dtype=torch.bfloat16, device=device), 1e-5)
+    with pytest.raises(HipAttnError, match="norm_weight must be"):
+        K.linear_rms_norm(xd, wd, nw[:512], 1e-5)
+
+
 def test_refusals(device):
     def t(*shape, dtype=torch.bfloat16):
         return torch.zeros(shape, dtype=dtype, device=device)
