@@ -1,6 +1,7 @@
-// Memory-system yardsticks for the benchmark: what this device delivers for a plain read, a copy, a fill and
-// a read of shuffled fixed-size chunks -- the figures the decode kernels' bandwidth is held against.  Built into
-// a library of its own (libmembench.so); nothing in the attention library links or calls it.
+// Yardsticks for the benchmark: what this device delivers for a plain read, a copy, a fill and a read of
+// shuffled fixed-size chunks -- the figures the decode kernels' bandwidth is held against -- and what its matrix
+// pipes deliver to a wavefront that does nothing but issue MFMAs, which the prefill kernels' rate is held
+// against.  Built into a library of its own (libmembench.so); nothing in the attention library links or calls it.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -59,7 +60,45 @@ __global__ __launch_bounds__(256) void read_chunks_kernel(const u32x4 *__restric
   }
   if (acc == 0x9e3779b9u && sink) sink[0] = acc;
 }
+
+// Every wavefront streams v_mfma_f32_32x32x16_bf16 into four independent accumulators: 16 x iters MFMAs per
+// wavefront, two wavefronts per SIMD, no memory traffic inside the loop.  The operands -- four A and four B
+// registers per lane, used in rotation -- come from `ops` (8 x 512 x 16 bytes), because what the card's power
+// management lets the pipes do depends on the values that flow through them.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+__global__ __launch_bounds__(512, 2) void mfma_stream_kernel(const u32x4 *__restrict__ ops, float *sink, int iters) {
+  bf16x8 a[4], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    a[i] = __builtin_bit_cast(bf16x8, ops[(2 * i) * 512 + threadIdx.x]);
+    b[i] = __builtin_bit_cast(bf16x8, ops[(2 * i + 1) * 512 + threadIdx.x]);
+  }
+  f32x16 c0 = {}, c1 = {}, c2 = {}, c3 = {};
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[i], c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(i + 1) & 3], b[i], c1, 0, 0, 0);
+      c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(i + 2) & 3], b[i], c2, 0, 0, 0);
+      c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(i + 3) & 3], b[i], c3, 0, 0, 0);
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; i++) s += c0[i] + c1[i] + c2[i] + c3[i];
+  if (s == 12345.678f && sink) sink[threadIdx.x] = s;  // (keeps the loop; never true by chance)
+}
 }  // namespace
+
+// One launch of the MFMA stream on `workgroups` workgroups of eight wavefronts: 16 * iters MFMAs of 32768 flop
+// per wavefront.  ops: 8 * 512 * 16 bytes of bf16 operands; sink may be null.  Returns 0, a hipError_t, or -1.
+extern "C" int membench_mfma_stream(const void *ops, void *sink, int workgroups, int iters, void *stream_arg) {
+  if (!ops || workgroups <= 0 || iters <= 0) return -1;
+  mfma_stream_kernel<<<workgroups, 512, 0, static_cast<hipStream_t>(stream_arg)>>>(static_cast<const u32x4 *>(ops),
+                                                                                  static_cast<float *>(sink), iters);
+  return (int)hipGetLastError();
+}
 
 // mode 0 reads src once (dst may be null), 1 copies src to dst, 2 fills dst, 3 reads the chunks of src that
 // chunks[0..n_chunks) number (each 0 <= chunks[k] < bytes / chunk_bytes; chunk_bytes a multiple of 4096);

@@ -1,6 +1,7 @@
-"""The benchmark's memory-system yardsticks (csrc/bench/membench.hip, built into libmembench.so): a plain read,
-a copy, a fill and a read of shuffled chunks on the device, for holding the decode kernels' bandwidth against
-what the part delivers.  Not part of the attention library and not used by it."""
+"""The benchmark's yardsticks (csrc/bench/membench.hip, built into libmembench.so): a plain read, a copy, a fill
+and a read of shuffled chunks on the device, for holding the decode kernels' bandwidth against what the part
+delivers, and a bare stream of MFMAs, for holding the prefill kernels' rate against what the matrix pipes deliver.
+Not part of the attention library and not used by it."""
 from __future__ import annotations
 
 import ctypes
@@ -22,7 +23,25 @@ def _load():
         _lib.membench_probe.restype = ctypes.c_int
         _lib.membench_probe.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
                                         ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+        _lib.membench_mfma_stream.restype = ctypes.c_int
+        _lib.membench_mfma_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
     return _lib
+
+
+MFMA_STREAM_OPERAND_ELEMS = 8 * 512 * 8  # bf16 elements that mfma_stream reads its operands from
+
+
+def mfma_stream(ops: torch.Tensor, workgroups: int, iters: int) -> float:
+    """One launch on torch's current stream of a kernel whose wavefronts (eight per workgroup, two per SIMD) do
+    nothing but issue v_mfma_f32_32x32x16_bf16 on the bf16 operands in `ops` (MFMA_STREAM_OPERAND_ELEMS elements);
+    returns the flops of the launch."""
+    if ops.dtype != torch.bfloat16 or ops.numel() < MFMA_STREAM_OPERAND_ELEMS or not ops.is_contiguous():
+        raise ValueError("mfma_stream: ops must be a contiguous bf16 tensor of MFMA_STREAM_OPERAND_ELEMS elements")
+    rc = _load().membench_mfma_stream(ops.data_ptr(), None, int(workgroups), int(iters),
+                                      ctypes.c_void_p(torch.cuda.current_stream(ops.device).cuda_stream))
+    if rc != 0:
+        raise RuntimeError(f"membench_mfma_stream failed with code {rc}")
+    return float(workgroups) * 8 * iters * 16 * 32768.0
 
 
 def probe(mode: str, dst: Optional[torch.Tensor], src: Optional[torch.Tensor], chunks: Optional[torch.Tensor] = None,

@@ -68,6 +68,105 @@ def spread(xs: list) -> dict:
             "max": round(max(xs), 5)}
 
 
+class PowerSampler:
+    """Reads the card's power (W) from the amdgpu hwmon files every 20 ms on a thread of its own, where the box
+    shows them; `mean(t0, t1)` is None where it does not."""
+
+    def __init__(self):
+        import glob
+
+        dirs = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))
+        self.file = next((os.path.join(d, "power1_input") for d in dirs if os.path.exists(os.path.join(d, "power1_input"))), None)
+        self.cap_w = None
+        if self.file:
+            try:
+                self.cap_w = int(open(os.path.join(os.path.dirname(self.file), "power1_cap")).read()) / 1e6
+            except (OSError, ValueError):
+                pass
+        self.samples, self._stop, self._thread = [], False, None
+
+    def _run(self):
+        while not self._stop:
+            try:
+                self.samples.append((time.perf_counter(), int(open(self.file).read()) / 1e6))
+            except (OSError, ValueError):
+                return
+            time.sleep(0.02)
+
+    def __enter__(self):
+        if self.file:
+            import threading
+
+            self._thread = threading.Thread(target=self._run, daemon=True)
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        if self._thread:
+            self._thread.join()
+
+    def mean(self, t0: float, t1: float):
+        xs = [w for (t, w) in self.samples if t0 <= t <= t1]
+        return round(sum(xs) / len(xs), 0) if xs else None
+
+
+def sustained(fn, seconds: float, est_ms: float, power: "PowerSampler") -> dict:
+    """`fn` back to back for about `seconds`: time per call over the whole run and the card's mean power over its
+    last two thirds.  Short timed runs start on a card that has been resting; this is what the same kernel does
+    once the card's power management has settled."""
+    import torch
+
+    n = max(50, int(seconds * 1e3 / est_ms))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n):
+        fn()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return {"launches": n, "ms_per_step": round((t1 - t0) * 1e3 / n, 4), "mean_power_w": power.mean(t0 + (t1 - t0) / 3, t1),
+            "power_cap_w": power.cap_w}
+
+
+def matrix_pipe_leg(dev, power: "PowerSampler") -> dict:
+    """What the matrix pipes of this card give a kernel that does nothing but issue v_mfma_f32_32x32x16_bf16 (two
+    wavefronts per SIMD on every compute unit, operands in registers), beside the published 2.5 PFLOP/s: after a
+    short warm-up as the prefill leg is timed, and sustained; with operands of ones and with N(0,1) operands like
+    the prefill leg's -- what the card's power management lets the pipes do depends on the values."""
+    import torch
+    from aici_amd import membench
+
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    iters = 2000  # 32000 MFMAs per wavefront and launch
+    out = {"kernel": "mfma_stream_kernel (csrc/bench/membench.hip), one workgroup of eight wavefronts per compute unit",
+           "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s"}
+    g = torch.Generator().manual_seed(23)
+    for name in ("ones", "normal"):
+        ops = (torch.ones(membench.MFMA_STREAM_OPERAND_ELEMS) if name == "ones"
+               else torch.randn(membench.MFMA_STREAM_OPERAND_ELEMS, generator=g)).to(torch.bfloat16).to(dev)
+        flop = [0.0]
+
+        def fn():
+            flop[0] = membench.mfma_stream(ops, cus, iters)
+
+        time.sleep(0.5)  # from a rested card, like the legs before it
+        for _ in range(25):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(50):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / 50
+        sus = sustained(fn, 1.5, ms, power)
+        out[f"operands_{name}"] = {
+            "after_25_launches": {"value": round(flop[0] / (ms * 1e-3) / 1e12, 1), "frac": round(flop[0] / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)},
+            "sustained": {**sus, "value": round(flop[0] / (sus["ms_per_step"] * 1e-3) / 1e12, 1),
+                          "frac": round(flop[0] / (sus["ms_per_step"] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}}
+    return out
+
+
 def host_cores() -> dict:
     """Cores this process may run on and cores the box reports (a container's share can be smaller); the CPU
     baselines run on every core the process may use, up to the thread count the box sets for such pools
@@ -537,6 +636,9 @@ def main() -> None:
                     help="skip the plain read / copy / fill kernels and the shuffled 4 KiB-chunk read (the "
                          "attainable rates reported beside the 8 TB/s peak)")
     ap.add_argument("--memory-system", action="store_true", help="(default; kept for old command lines)")
+    ap.add_argument("--no-sustained", action="store_true",
+                    help="skip the runs of about 1.5 s each (prefill, and a bare stream of MFMAs) that show what the card "
+                         "holds once its power management has settled, with the card's power beside them")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (torch copy_) so that FETCH_SIZE / WRITE_SIZE "
                          "read under rocprofv3 --pmc can be scaled against a kernel of known traffic")
@@ -622,6 +724,13 @@ def main() -> None:
         "host_cores": host_cores(),
     }
 
+    if not args.no_sustained:
+        # the same step for about a second, with the card's power beside it (a memory-bound step leaves the card
+        # well inside its power limit; the prefill leg below does not)
+        with PowerSampler() as power:
+            sus = sustained(decode_step, 1.0, avg_step_ms, power)
+        line["roofline"]["sustained"] = {**sus, "achieved": round(nbytes / (sus["ms_per_step"] * 1e-3) / 1e9, 1),
+                                         "frac": round(nbytes / (sus["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     if args.copy_calibration:
         src = torch.empty((1 << 30,), dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
@@ -658,6 +767,14 @@ def main() -> None:
                          "kernel": "prefill_varlen_w8_kernel, HIP events on the launch stream",
                          "avg_launch_us": round(pms * 1e3, 1)},
         }
+        if not args.no_sustained:
+            # ... and once the card's power management has settled: about 1.5 s of launches back to back
+            with PowerSampler() as power:
+                sus = sustained(prefill_step, 1.5, pms, power)
+            sus_tf = p.flops() / (sus["ms_per_step"] * 1e-3) / 1e12
+            line["prefill"]["sustained"] = {**sus, "value": round(sus_tf, 1), "unit": "TFLOP/s",
+                                            "frac": round(sus_tf / MFMA_BF16_PEAK_TFLOPS, 4)}
+            time.sleep(0.5)
         # The same rows with K/V read from the paged cache they were scattered into (what an engine step
         # has at hand: rLLM writes the cache first, llm/mod.rs:147-164, and gathers back from it).
         nb = sum((l + 15) // 16 for l in p.lens_k)
@@ -714,6 +831,10 @@ def main() -> None:
                     "kernel": "prefill_varlen_r3_kernel (prefill_kernel = 4)", "ms_per_step": round(rms, 4),
                     "value": round(p.flops() / (rms * 1e-3) / 1e12, 1), "unit": "TFLOP/s"}}
             del p
+
+        if not args.no_sustained:
+            with PowerSampler() as power:
+                line["prefill"]["matrix_pipe"] = matrix_pipe_leg(dev, power)
 
     # ---- optional: the streaming helpers -------------------------------------------------------------
     if args.streaming:

@@ -412,3 +412,19 @@ def test_memory_yardsticks_of_the_benchmark(device):
         membench.probe("read", None, src[:100])
     with pytest.raises(RuntimeError, match="bad arguments"):
         membench.probe("read_chunks", None, src[: 4096 + 16], chunks)
+
+
+def test_matrix_pipe_yardstick_of_the_benchmark(device):
+    """The benchmark's bare stream of MFMAs launches, counts its flops as 16 x iters MFMAs of 32 x 32 x 16 per
+    wavefront, leaves its operands alone and refuses operands of another kind."""
+    from aici_amd import membench
+    ops = torch.randn(membench.MFMA_STREAM_OPERAND_ELEMS, generator=torch.Generator().manual_seed(6)).to(torch.bfloat16).to(device)
+    before = ops.cpu().clone()
+    flop = membench.mfma_stream(ops, 4, 10)
+    torch.cuda.synchronize()
+    assert flop == 4 * 8 * 10 * 16 * 2 * 32 * 32 * 16
+    assert torch.equal(ops.cpu().view(torch.int16), before.view(torch.int16))
+    with pytest.raises(ValueError):
+        membench.mfma_stream(ops.float(), 4, 10)
+    with pytest.raises(ValueError):
+        membench.mfma_stream(ops[:100], 4, 10)
