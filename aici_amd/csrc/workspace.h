@@ -30,7 +30,7 @@ struct Tuning {
   int prefill_kernel;      // 0: the library chooses; 1: eight wavefronts; 2 / 3: four wavefronts, 2 / 1 row tiles each; 4: three groups of four
   int paged_prefill_dma;   // -1: the library chooses; 0: staged tiles; 1: block images where possible
   int cache_move_lds;      // -1: the library chooses; 0: never the LDS-transposing kernels
-  int prefill_wg_heads;      // eight-wavefront prefill: query heads of one kv group per workgroup, at most (0 and 1: one)
+  int prefill_wg_heads;      // eight-wavefront prefill: query heads of one kv group per workgroup, at most (0: the library chooses -- up to four; 1: one)
   int prefill_rescale_log2;  // prefill: a row's reference maximum moves when outgrown by more than 2^this (0..16, default 8)
   int linear_tiles;          // linear: 16-row tiles of the weight per wavefront (0: the library chooses; 1 or 2)
   int linear_waves;          // linear: wavefronts per workgroup (0: the library chooses; 4 or 8)

@@ -484,7 +484,8 @@ char *hipattn_shutdown(void);
  * wavefronts), paged_prefill_dma (-1 library's
  * choice, 0 staged tiles), cache_move_lds (-1 library's choice, 0 never the
  * LDS-transposing kernels), prefill_wg_heads (query heads of one kv group per
- * workgroup of the eight-wavefront prefill kernel, at most; 0 and 1: one),
+ * workgroup of the eight-wavefront prefill kernel, at most; 0 library's
+ * choice -- up to four -- 1: one),
  * prefill_rescale_log2 (0..16, default 8: the prefill
  * kernels move a row's reference maximum only when the row outgrows it by
  * more than 2^value; 0 follows the row maximum exactly, as the reference
