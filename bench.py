@@ -34,8 +34,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
 PROFILED = {
     "decode_traffic_bytes": 642.7e6,      # FETCH_SIZE + WRITE_SIZE per decode step, scaled by a 1 GiB copy
     "decode_traffic_source": "profiles/decode_c2_prefill_c3_hbm_traffic.md",
-    "decode_main_kernel_us": 101.7,       # paged_decode_flat_kernel, average duration in the kernel trace
-    "decode_reduce_kernel_us": 4.9,       # paged_decode_flat_reduce_kernel
+    "decode_main_kernel_us": 101.9,       # paged_decode_flat_kernel, average duration in the kernel trace
+    "decode_reduce_kernel_us": 4.7,       # paged_decode_flat_reduce_kernel
     "decode_kernels_source": "profiles/decode_c2_prefill_c3_kernel_trace.md",
     "prefill_traffic_bytes": 671.4e6,     # FETCH_SIZE + WRITE_SIZE per prefill launch, same scaling
     "prefill_traffic_source": "profiles/decode_c2_prefill_c3_hbm_traffic.md",
